@@ -1,0 +1,211 @@
+// C ABI of libaeris_hip.so: argument validation (host only, before any GPU call), error reporting,
+// one-time kernel attribute set-up, and the host-side index-map test hooks.
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(AERIS_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+std::once_flag g_init_once;
+hipError_t g_init_status = hipSuccess;
+
+int ensure_init() {
+  std::call_once(g_init_once, [] {
+    g_init_status = aeris::gemm_configure_all();
+    if (g_init_status == hipSuccess) g_init_status = aeris::attention_configure_all();
+  });
+  if (g_init_status != hipSuccess) return hip_fail(g_init_status, "aeris_init (hipFuncSetAttribute)");
+  return AERIS_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_window_geometry(int B, int H, int W, int ws_y, int ws_x, int shift_y, int shift_x) {
+  if (B <= 0 || H <= 0 || W <= 0 || ws_y <= 0 || ws_x <= 0)
+    return fail(AERIS_EINVAL, "window geometry: B, H, W, ws_y, ws_x must be positive (got %d %d %d %d %d)", B, H, W, ws_y, ws_x);
+  if (H % ws_y || W % ws_x)
+    return fail(AERIS_EINVAL, "window geometry: grid %dx%d is not a multiple of window %dx%d", H, W, ws_y, ws_x);
+  if (shift_y < 0 || shift_x < 0 || shift_y >= ws_y || shift_x >= ws_x)
+    return fail(AERIS_EINVAL, "window geometry: shift (%d,%d) must lie in [0, window)", shift_y, shift_x);
+  return AERIS_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int aeris_version(void) { return 1; }
+
+const char* aeris_last_error(void) { return g_err; }
+
+int aeris_init(void) { return ensure_init(); }
+
+int aeris_window_index_map(int B, int H, int W, int ws_y, int ws_x, int shift_y, int shift_x, int64_t* out) {
+  if (!out) return fail(AERIS_EINVAL, "aeris_window_index_map: out is NULL");
+  if (int rc = check_window_geometry(B, H, W, ws_y, ws_x, shift_y, shift_x)) return rc;
+  const int nWy = H / ws_y, nWx = W / ws_x;
+  int64_t o = 0;
+  for (int b = 0; b < B; ++b)
+    for (int wy = 0; wy < nWy; ++wy)
+      for (int wx = 0; wx < nWx; ++wx) {
+        // same arithmetic as token_row() of the attention kernel
+        const int y0 = wy * ws_y + shift_y, x0 = wx * ws_x + shift_x;
+        for (int pos = 0; pos < ws_y * ws_x; ++pos) {
+          int Y = y0 + pos / ws_x, X = x0 + pos % ws_x;
+          if (Y >= H) Y -= H;
+          if (X >= W) X -= W;
+          out[o++] = (int64_t)b * H * W + (int64_t)Y * W + X;
+        }
+      }
+  return AERIS_OK;
+}
+
+int aeris_relative_position_index(int ws_y, int ws_x, int32_t* out) {
+  if (!out) return fail(AERIS_EINVAL, "aeris_relative_position_index: out is NULL");
+  if (ws_y <= 0 || ws_x <= 0) return fail(AERIS_EINVAL, "aeris_relative_position_index: window must be positive");
+  const int L = ws_y * ws_x;
+  for (int p = 0; p < L; ++p)
+    for (int q = 0; q < L; ++q) {
+      // same closed form as the kernel: (iy_p - iy_q + ws_y - 1) * (2 ws_x - 1) + (ix_p - ix_q + ws_x - 1)
+      const int dy = p / ws_x - q / ws_x + ws_y - 1;
+      const int dx = p % ws_x - q % ws_x + ws_x - 1;
+      out[p * L + q] = dy * (2 * ws_x - 1) + dx;
+    }
+  return AERIS_OK;
+}
+
+int aeris_shift_region_ids(int H, int W, int ws_y, int ws_x, int shift_y, int shift_x, int32_t* out) {
+  if (!out) return fail(AERIS_EINVAL, "aeris_shift_region_ids: out is NULL");
+  if (int rc = check_window_geometry(1, H, W, ws_y, ws_x, shift_y, shift_x)) return rc;
+  const int nWy = H / ws_y, nWx = W / ws_x;
+  int64_t o = 0;
+  for (int wy = 0; wy < nWy; ++wy)
+    for (int wx = 0; wx < nWx; ++wx) {
+      const bool my = shift_y > 0 && wy == nWy - 1;
+      const bool mx = shift_x > 0 && wx == nWx - 1;
+      for (int iy = 0; iy < ws_y; ++iy)
+        for (int ix = 0; ix < ws_x; ++ix) {
+          // same predicate as the kernel's mask pass
+          const int ry = my ? (iy < ws_y - shift_y ? 1 : 2) : 0;
+          const int rx = mx ? (ix < ws_x - shift_x ? 1 : 2) : 0;
+          out[o++] = 3 * ry + rx;
+        }
+    }
+  return AERIS_OK;
+}
+
+int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
+                               int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
+                               void* stream) {
+  if (!qkv || !out) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: qkv/out is NULL");
+  if (!aligned16(qkv) || !aligned16(out)) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: qkv/out must be 16-byte aligned");
+  if (heads <= 0 || head_dim <= 0) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: heads/head_dim must be positive");
+  if (int rc = check_window_geometry(B, H, W, ws_y, ws_x, shift_y, shift_x)) return rc;
+  if (!(scale > 0.f)) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: scale must be positive");
+  if (!aeris::attention_supported(ws_y, ws_x, head_dim))
+    return fail(AERIS_EUNSUPPORTED,
+                "aeris_window_attention_fwd: no kernel for window %dx%d head_dim %d (built: 8x8, 12x12, 16x16 with head_dim 32 or 64)",
+                ws_y, ws_x, head_dim);
+  if ((int64_t)B * (H / ws_y) * (W / ws_x) * heads > 0x7fffffffLL)
+    return fail(AERIS_EUNSUPPORTED, "aeris_window_attention_fwd: more than 2^31-1 (window, head) pairs");
+  if (int rc = ensure_init()) return rc;
+  hipError_t e = aeris::attention_launch(qkv, out, bias_table, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x,
+                                         use_mask, scale, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_window_attention_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,
+                            int param_dtype, const float* shift, const float* scale, int64_t mod_batch_stride, int64_t B,
+                            int64_t rows_per_batch, int d, int kind, int order, float eps, void* stream) {
+  if (!x || !y || !gamma) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: x/y/gamma is NULL");
+  if (!aligned16(x) || !aligned16(y)) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: x/y must be 16-byte aligned");
+  if (B <= 0 || rows_per_batch <= 0) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: B and rows_per_batch must be positive");
+  if ((x_dtype != AERIS_BF16 && x_dtype != AERIS_F32) || (y_dtype != AERIS_BF16 && y_dtype != AERIS_F32) ||
+      (param_dtype != AERIS_BF16 && param_dtype != AERIS_F32))
+    return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: dtype must be AERIS_BF16 or AERIS_F32");
+  if (kind != AERIS_NORM_LAYER && kind != AERIS_NORM_RMS) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: unknown norm kind %d", kind);
+  if (order != AERIS_NORM_THEN_MOD && order != AERIS_MOD_THEN_NORM) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: unknown order %d", order);
+  if (mod_batch_stride < 0) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: negative mod_batch_stride");
+  if (!(eps >= 0.f)) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: eps must be non-negative");
+  if (!aeris::norm_supported(d)) return fail(AERIS_EUNSUPPORTED, "aeris_norm_modulate_fwd: d=%d (need d %% 8 == 0 and d <= 6144)", d);
+  hipError_t e = aeris::norm_modulate_launch(x, x_dtype, y, y_dtype, gamma, beta, param_dtype, shift, scale, mod_batch_stride, B,
+                                             rows_per_batch, d, kind, order, eps, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_norm_modulate_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, const float* gate, const void* residual,
+                   int64_t M, int N, int K, int64_t ldc, int act, int res_dtype, int c_dtype,
+                   int64_t gate_batch_stride, int64_t rows_per_batch, void* stream) {
+  if (!A || !W || !C) return fail(AERIS_EINVAL, "aeris_gemm_fwd: A/W/C is NULL");
+  if (M <= 0 || N <= 0 || K <= 0) return fail(AERIS_EINVAL, "aeris_gemm_fwd: M, N, K must be positive");
+  if (!aligned16(A) || !aligned16(W) || !aligned16(C) || (residual && !aligned16(residual)))
+    return fail(AERIS_EINVAL, "aeris_gemm_fwd: A/W/C/residual must be 16-byte aligned");
+  if (K % 64) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_fwd: K=%d must be a multiple of 64", K);
+  if (ldc < N) return fail(AERIS_EINVAL, "aeris_gemm_fwd: ldc < N");
+  if (act < AERIS_ACT_NONE || act > AERIS_ACT_SILU) return fail(AERIS_EINVAL, "aeris_gemm_fwd: unknown activation %d", act);
+  if (c_dtype != AERIS_BF16 && c_dtype != AERIS_F32) return fail(AERIS_EINVAL, "aeris_gemm_fwd: bad c_dtype");
+  if (residual && res_dtype != AERIS_BF16 && res_dtype != AERIS_F32) return fail(AERIS_EINVAL, "aeris_gemm_fwd: bad res_dtype");
+  if (gate && gate_batch_stride && rows_per_batch <= 0)
+    return fail(AERIS_EINVAL, "aeris_gemm_fwd: rows_per_batch must be positive with a per-batch gate");
+  if (gate_batch_stride < 0) return fail(AERIS_EINVAL, "aeris_gemm_fwd: negative gate_batch_stride");
+  if ((int64_t)((M + 127) / 128) * ((N + 63) / 64) > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_fwd: too many tiles");
+  if (int rc = ensure_init()) return rc;
+  hipError_t e = aeris::gemm_launch(A, W, C, bias, gate, residual, M, N, K, ldc, act, res_dtype, c_dtype,
+                                    gate_batch_stride, rows_per_batch, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_gemm_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_modulation_linear_fwd(const float* x, const void* W, const void* bias, float* y, int B, int N, int K,
+                                int w_dtype, int act, void* stream) {
+  if (!x || !W || !y) return fail(AERIS_EINVAL, "aeris_modulation_linear_fwd: x/W/y is NULL");
+  if (B <= 0 || N <= 0 || K <= 0) return fail(AERIS_EINVAL, "aeris_modulation_linear_fwd: B, N, K must be positive");
+  if (K % 8) return fail(AERIS_EUNSUPPORTED, "aeris_modulation_linear_fwd: K=%d must be a multiple of 8", K);
+  if (!aligned16(x) || !aligned16(W)) return fail(AERIS_EINVAL, "aeris_modulation_linear_fwd: x/W must be 16-byte aligned");
+  if (w_dtype != AERIS_BF16 && w_dtype != AERIS_F32) return fail(AERIS_EINVAL, "aeris_modulation_linear_fwd: bad w_dtype");
+  if (act != AERIS_ACT_NONE && act != AERIS_ACT_SILU) return fail(AERIS_EINVAL, "aeris_modulation_linear_fwd: act must be NONE or SILU");
+  hipError_t e = aeris::modulation_linear_launch(x, W, bias, y, B, N, K, w_dtype, act, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_modulation_linear_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_timestep_embedding_fwd(const float* t, float* emb, int B, int dim, float max_period, void* stream) {
+  if (!t || !emb) return fail(AERIS_EINVAL, "aeris_timestep_embedding_fwd: t/emb is NULL");
+  if (B <= 0 || dim <= 0 || dim % 2) return fail(AERIS_EINVAL, "aeris_timestep_embedding_fwd: B > 0 and even dim > 0 required");
+  if (!(max_period > 1.f)) return fail(AERIS_EINVAL, "aeris_timestep_embedding_fwd: max_period must exceed 1");
+  hipError_t e = aeris::timestep_embedding_launch(t, emb, B, dim, max_period, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_timestep_embedding_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_embed_prepare_fwd(const float* x, const float* ape, void* out, int64_t M, int64_t M_ape, int C, int K_pad,
+                            void* stream) {
+  if (!x || !out) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: x/out is NULL");
+  if (M <= 0 || C <= 0 || K_pad < C || K_pad % 64) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: need M > 0, 0 < C <= K_pad, K_pad %% 64 == 0");
+  if (ape && M_ape <= 0) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: M_ape must be positive when ape is given");
+  if (!aligned16(out)) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: out must be 16-byte aligned");
+  hipError_t e = aeris::embed_prepare_launch(x, ape, out, M, M_ape > 0 ? M_ape : 1, C, K_pad, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_embed_prepare_fwd launch");
+  return AERIS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,307 @@
+// bf16 MFMA GEMM for gfx950:  C[M,N] = epilogue(A[M,K] * W[N,K]^T)
+//
+// Both operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_bf16 wants for its
+// A and B fragments (8 consecutive k per lane).  One workgroup computes a BM x BN tile of C:
+//   - global -> registers -> LDS with a one-tile look-ahead, two LDS stages, one barrier per k-tile
+//   - LDS rows are 128 B (64 bf16) and 16-byte chunks are XOR-swizzled over a 256 B double row so
+//     that both the ds_write_b128 of the loader and the ds_read_b128 of the fragment reads spread
+//     over all banks
+//   - the weight fragment is the first MFMA operand, so a lane ends up with 4 consecutive n for
+//     one m and the epilogue stores 8 B (bf16) / 16 B (f32) vectors
+//   - blockIdx is remapped so that each XCD (blockIdx % 8) works on a contiguous range of tiles,
+//     n fastest, which keeps the A row panels of a range in that XCD's L2
+// Epilogue (all optional, fused): + bias[n], GELU / SiLU / SwiGLU, * gate[b, n], + residual[m, n].
+#include "common.h"
+#include "kernels.h"
+
+namespace aeris {
+
+struct GemmParams {
+  const uint16_t* A;
+  const uint16_t* W;
+  void* C;
+  const uint16_t* bias;
+  const float* gate;
+  const void* residual;
+  int64_t M;
+  int N;  // logical output columns
+  int K;
+  int64_t ldc;
+  int64_t gate_batch_stride;
+  int64_t rows_per_batch;
+  int tiles_n;
+  int act;
+  int res_dtype;  // -1 none, AERIS_BF16, AERIS_F32
+  int c_dtype;
+};
+
+__device__ __forceinline__ uint32_t swz_off(int row, int chunk) {
+  // byte offset of 16-byte chunk `chunk` (0..7) of tile row `row` in a [rows][64] bf16 tile
+  return (uint32_t)((row >> 1) * 256 + (((((row & 1) << 3) | chunk) ^ ((row >> 1) & 7)) << 4));
+}
+
+template <int BM, int BN, int WM, int WN, bool SWIGLU, bool VEC>
+__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_nt_kernel(GemmParams p) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int BK = 64;
+  constexpr int FM = BM / WM / 32;
+  constexpr int FN = BN / WN / 32;
+  constexpr int A_BYTES = BM * BK * 2;
+  constexpr int B_BYTES = BN * BK * 2;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  constexpr int RP = NT / 8;  // tile rows covered by one pass of the loader
+  constexpr int A_IT = BM / RP;
+  constexpr int B_IT = BN / RP;
+  static_assert(!SWIGLU || FN == 2, "SwiGLU pairs fragment 0 (gate) with fragment 1 (up)");
+  static_assert(RP % 16 == 0, "swizzle phase must repeat across loader passes");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  // ---- tile selection with XCD-contiguous remap
+  const int np = gridDim.x;
+  int pid = blockIdx.x;
+  {
+    const int per = (np + 7) >> 3;
+    int tall = np & 7;
+    if (tall == 0) tall = 8;
+    const int xcd = pid & 7, loc = pid >> 3;
+    pid = (xcd < tall) ? xcd * per + loc : tall * per + (xcd - tall) * (per - 1) + loc;
+  }
+  const int tile_m = pid / p.tiles_n;
+  const int tile_n = pid - tile_m * p.tiles_n;
+  const int64_t m0 = (int64_t)tile_m * BM;
+  constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
+  const int n0 = tile_n * BN_OUT;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int l31 = lane & 31, hi = lane >> 5;
+
+  // ---- loader mapping: thread -> (row lr + i*RP, chunk lc)
+  const int lc = tid & 7, lr = tid >> 3;
+  const int K = p.K;
+  uint32_t a_goff[A_IT], b_goff[B_IT];  // element offsets from the tile's first row
+  const uint16_t* a_base;
+  const uint16_t* b_base;
+  {
+    const int64_t last = p.M - 1 - m0;  // >= 0
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+      int64_t r = lr + i * RP;
+      if (r > last) r = last;
+      a_goff[i] = (uint32_t)(r * K + lc * 8);
+    }
+    a_base = p.A + m0 * K;
+    const int wrows = SWIGLU ? 2 * p.N : p.N;
+    int first_row;
+    if (SWIGLU) first_row = 0; else first_row = n0;
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) {
+      const int j = lr + i * RP;  // tile row
+      int r;
+      if (SWIGLU) {
+        constexpr int WNW = BN / WN;  // tile columns owned by one wave: [gate 32 | up 32]
+        const int wv = j / WNW, within = j % WNW;
+        const int oc = n0 + wv * 32 + (within & 31);
+        r = ((within >> 5) ? p.N : 0) + (oc < p.N ? oc : p.N - 1);
+      } else {
+        r = n0 + j;
+        if (r > wrows - 1) r = wrows - 1;
+        r -= first_row;
+      }
+      b_goff[i] = (uint32_t)((int64_t)r * K + lc * 8);
+    }
+    b_base = p.W + (int64_t)first_row * K;
+  }
+  const uint32_t w_off = swz_off(lr, lc);
+
+  // ---- fragment read offsets (per k16 step)
+  uint32_t a_roff[4], b_roff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    a_roff[ks] = swz_off(wm * (BM / WM) + l31, ks * 2 + hi);
+    b_roff[ks] = A_BYTES + swz_off(wn * (BN / WN) + l31, ks * 2 + hi);
+  }
+
+  f32x16 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  u32x4 ra[A_IT], rb[B_IT];
+  auto gload = [&](int kt) {
+    const uint16_t* ab = a_base + (int64_t)kt * BK;
+    const uint16_t* bb = b_base + (int64_t)kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab + a_goff[i]);
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) rb[i] = *reinterpret_cast<const u32x4*>(bb + b_goff[i]);
+  };
+  auto lstore = [&](int stage) {
+    unsigned char* s = smem + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) *reinterpret_cast<u32x4*>(s + w_off + i * RP * 128) = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) *reinterpret_cast<u32x4*>(s + A_BYTES + w_off + i * RP * 128) = rb[i];
+  };
+
+  const int KT = K / BK;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const bool more = kt + 1 < KT;
+    if (more) gload(kt + 1);
+    const unsigned char* s = smem + (kt & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      bf16x8 af[FM], bfr[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(s + a_roff[ks] + i * 32 * 128);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) bfr[j] = *reinterpret_cast<const bf16x8*>(s + b_roff[ks] + j * 32 * 128);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+    }
+    if (more) lstore((kt + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds, per (i, j, g), 4 consecutive n for row m
+  const int N = p.N;
+  constexpr int FN_OUT = SWIGLU ? 1 : FN;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int64_t m = m0 + wm * (BM / WM) + i * 32 + l31;
+    const bool m_ok = m < p.M;
+    const float* gate_row = nullptr;
+    if (p.gate) gate_row = p.gate + (p.gate_batch_stride ? (m / p.rows_per_batch) * p.gate_batch_stride : 0);
+#pragma unroll
+    for (int j = 0; j < FN_OUT; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = SWIGLU ? n0 + wn * 32 + g * 8 + hi * 4 : n0 + wn * (BN / WN) + j * 32 + g * 8 + hi * 4;
+        if (m_ok && n < N) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int nn = (n + e < N) ? n + e : N - 1;
+          float x = acc[i][j][g * 4 + e];
+          if (SWIGLU) {
+            float u = acc[i][1][g * 4 + e];
+            if (p.bias) {
+              x += bf16_bits_to_f32(p.bias[nn]);
+              u += bf16_bits_to_f32(p.bias[N + nn]);
+            }
+            x = silu_f(x) * u;
+          } else {
+            if (p.bias) x += bf16_bits_to_f32(p.bias[nn]);
+            if (p.act == AERIS_ACT_GELU) x = gelu_erf_f(x);
+            else if (p.act == AERIS_ACT_SILU) x = silu_f(x);
+          }
+          if (gate_row) x *= gate_row[nn];
+          v[e] = x;
+        }
+        const int64_t off = m * p.ldc + n;
+        if (VEC) {
+          if (p.res_dtype == AERIS_BF16) {
+            const u32x2 r = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
+            v[0] += bf16_lo(r.x); v[1] += bf16_hi(r.x); v[2] += bf16_lo(r.y); v[3] += bf16_hi(r.y);
+          } else if (p.res_dtype == AERIS_F32) {
+            const f32x4 r = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.residual) + off);
+            v[0] += r.x; v[1] += r.y; v[2] += r.z; v[3] += r.w;
+          }
+          if (p.c_dtype == AERIS_BF16) {
+            u32x2 o;
+            o.x = pack_bf16x2(v[0], v[1]);
+            o.y = pack_bf16x2(v[2], v[3]);
+            *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(p.C) + off) = o;
+          } else {
+            f32x4 o = {v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + off) = o;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (n + e < N) {
+            float x = v[e];
+            if (p.res_dtype == AERIS_BF16) x += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.residual)[off + e]);
+            else if (p.res_dtype == AERIS_F32) x += reinterpret_cast<const float*>(p.residual)[off + e];
+            if (p.c_dtype == AERIS_BF16) reinterpret_cast<uint16_t*>(p.C)[off + e] = (uint16_t)f32_to_bf16_bits(x);
+            else reinterpret_cast<float*>(p.C)[off + e] = x;
+            }
+          }
+        }
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN, bool SWIGLU, bool VEC>
+static hipError_t launch_gemm(const GemmParams& p0, hipStream_t stream) {
+  GemmParams p = p0;
+  constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
+  const int64_t tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+  const int64_t grid = tiles_m * p.tiles_n;
+  constexpr int smem = 2 * (BM + BN) * 64 * 2;
+  auto kern = gemm_bf16_nt_kernel<BM, BN, WM, WN, SWIGLU, VEC>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WM * WN * 64), smem, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gemm_configure_all() {
+  // touch every instantiation so that attribute set-up never happens inside a captured region
+  hipError_t e;
+#define CFG(BM, BN, WM, WN, SG, VC)                                                                          \
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_kernel<BM, BN, WM, WN, SG, VC>),          \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, 2 * (BM + BN) * 64 * 2);                 \
+  if (e != hipSuccess) return e;
+  CFG(256, 256, 2, 4, false, true)
+  CFG(256, 256, 2, 4, true, true)
+  CFG(128, 128, 2, 2, false, true)
+  CFG(128, 128, 2, 2, true, true)
+  CFG(128, 128, 2, 2, false, false)
+  CFG(128, 128, 2, 2, true, false)
+#undef CFG
+  return hipSuccess;
+}
+
+hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, const float* gate,
+                       const void* residual, int64_t M, int N, int K, int64_t ldc, int act, int res_dtype,
+                       int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, hipStream_t stream) {
+  GemmParams p;
+  p.A = reinterpret_cast<const uint16_t*>(A);
+  p.W = reinterpret_cast<const uint16_t*>(W);
+  p.C = C;
+  p.bias = reinterpret_cast<const uint16_t*>(bias);
+  p.gate = gate;
+  p.residual = residual;
+  p.M = M; p.N = N; p.K = K; p.ldc = ldc;
+  p.gate_batch_stride = gate_batch_stride;
+  p.rows_per_batch = rows_per_batch > 0 ? rows_per_batch : M;
+  p.tiles_n = 0;
+  p.act = act;
+  p.res_dtype = residual ? res_dtype : -1;
+  p.c_dtype = c_dtype;
+  const bool swiglu = act == AERIS_ACT_SWIGLU;
+  // big tiles when they are not mostly padding and there are enough of them to fill 256 CUs
+  const int bn_out = swiglu ? 128 : 256;
+  const bool big = (M >= 256) && (N % bn_out == 0 || N >= 4 * bn_out) &&
+                   ((M + 255) / 256) * ((N + bn_out - 1) / bn_out) >= 256;
+  // vector epilogue (8 / 16 byte accesses to C and the residual) needs 4-element alignment of every row
+  const bool vec = ((ldc & 3) == 0) && ((N & 3) == 0);
+  if (!vec) return swiglu ? launch_gemm<128, 128, 2, 2, true, false>(p, stream) : launch_gemm<128, 128, 2, 2, false, false>(p, stream);
+  if (swiglu) return big ? launch_gemm<256, 256, 2, 4, true, true>(p, stream) : launch_gemm<128, 128, 2, 2, true, true>(p, stream);
+  return big ? launch_gemm<256, 256, 2, 4, false, true>(p, stream) : launch_gemm<128, 128, 2, 2, false, true>(p, stream);
+}
+
+}  // namespace aeris

@@ -1,0 +1,34 @@
+// Internal launch interface between the C-ABI layer (api.hip) and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/aeris_hip.h"
+
+namespace aeris {
+
+// one-time hipFuncSetAttribute(MaxDynamicSharedMemorySize) for every kernel that needs > 64 KB LDS
+hipError_t gemm_configure_all();
+hipError_t attention_configure_all();
+
+hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, const float* gate,
+                       const void* residual, int64_t M, int N, int K, int64_t ldc, int act, int res_dtype,
+                       int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, hipStream_t stream);
+
+// returns hipErrorInvalidValue when (ws_y, ws_x, head_dim) has no instantiation
+bool attention_supported(int ws_y, int ws_x, int head_dim);
+hipError_t attention_launch(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
+                            int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
+                            hipStream_t stream);
+
+bool norm_supported(int d);
+hipError_t norm_modulate_launch(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,
+                                int param_dtype, const float* shift, const float* scale, int64_t mod_batch_stride, int64_t B,
+                                int64_t rows_per_batch, int d, int kind, int order, float eps, hipStream_t stream);
+
+hipError_t modulation_linear_launch(const float* x, const void* W, const void* bias, float* y, int B, int N, int K,
+                                    int w_dtype, int act, hipStream_t stream);
+hipError_t timestep_embedding_launch(const float* t, float* emb, int B, int dim, float max_period, hipStream_t stream);
+hipError_t embed_prepare_launch(const float* x, const float* ape, void* out, int64_t M, int64_t M_ape, int C, int K_pad,
+                                hipStream_t stream);
+
+}  // namespace aeris

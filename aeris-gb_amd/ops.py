@@ -1,0 +1,213 @@
+"""Tensor-level wrappers over the C ABI: check tensors, pass raw pointers and the current HIP stream.
+
+torch is used for device memory and streams only; all arithmetic happens in libaeris_hip.so.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib as L
+
+_DT = {torch.bfloat16: L.BF16, torch.float32: L.F32}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (the HIP kernels have no CPU fallback)")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
+    return t
+
+
+# ------------------------------------------------------------------------------------------
+# host-only index maps (no GPU needed)
+
+def window_index_map(B, H, W, ws_y, ws_x, shift_y=0, shift_x=0) -> np.ndarray:
+    if min(B, H, W, ws_y, ws_x) <= 0 or H % ws_y or W % ws_x:
+        n = 1
+    else:
+        n = B * H * W
+    out = np.empty(n, dtype=np.int64)
+    L.call("aeris_window_index_map", B, H, W, ws_y, ws_x, shift_y, shift_x, out.ctypes.data)
+    return out.reshape(B * (H // ws_y) * (W // ws_x), ws_y * ws_x)
+
+
+def relative_position_index(ws_y, ws_x) -> np.ndarray:
+    n = max(1, ws_y * ws_x)
+    out = np.empty(n * n, dtype=np.int32)
+    L.call("aeris_relative_position_index", ws_y, ws_x, out.ctypes.data)
+    return out.reshape(n, n)
+
+
+def shift_region_ids(H, W, ws_y, ws_x, shift_y, shift_x) -> np.ndarray:
+    ok = min(H, W, ws_y, ws_x) > 0 and H % ws_y == 0 and W % ws_x == 0
+    out = np.empty(H * W if ok else 1, dtype=np.int32)
+    L.call("aeris_shift_region_ids", H, W, ws_y, ws_x, shift_y, shift_x, out.ctypes.data)
+    return out.reshape((H // ws_y) * (W // ws_x), ws_y * ws_x)
+
+
+# ------------------------------------------------------------------------------------------
+# device ops
+
+def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], heads: int, head_dim: int,
+                     window_size: Tuple[int, int], shift: Tuple[int, int] = (0, 0),
+                     bias_table: Optional[torch.Tensor] = None, use_mask: bool = False,
+                     scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """qkv bf16 [B*H*W, 3*heads*head_dim] (natural token order) -> bf16 [B*H*W, heads*head_dim]."""
+    H, W = image_shape
+    inner = heads * head_dim
+    _dev(qkv, "qkv", torch.bfloat16)
+    if qkv.numel() != B * H * W * 3 * inner:
+        raise RuntimeError(f"qkv has {qkv.numel()} elements, expected {B}*{H}*{W}*3*{inner}")
+    if bias_table is not None:
+        _dev(bias_table, "bias_table", torch.bfloat16)
+        n = (2 * window_size[0] - 1) * (2 * window_size[1] - 1)
+        if tuple(bias_table.shape) != (n, heads):
+            raise RuntimeError(f"bias_table must be [{n}, {heads}], got {tuple(bias_table.shape)}")
+    if out is None:
+        out = torch.empty(B * H * W, inner, dtype=torch.bfloat16, device=qkv.device)
+    else:
+        _dev(out, "out", torch.bfloat16)
+        if out.numel() != B * H * W * inner:
+            raise RuntimeError("out has the wrong size")
+    L.call("aeris_window_attention_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads, head_dim,
+           window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
+           float(head_dim ** -0.5 if scale is None else scale), _stream())
+    return out
+
+
+def _rowvec(t: Optional[torch.Tensor], name: str, d: int, B: int):
+    """f32 [1|B, d] row vectors, rows possibly strided (a chunk of a wider matrix): -> (ptr, batch stride)."""
+    if t is None:
+        return None, 0
+    if not t.is_cuda or t.dtype != torch.float32:
+        raise RuntimeError(f"{name} must be a float32 GPU tensor")
+    if t.dim() != 2 or t.shape[1] != d or t.stride(1) != 1 or t.shape[0] not in (1, B):
+        raise RuntimeError(f"{name} must be [1, {d}] or [{B}, {d}] with unit column stride, got {tuple(t.shape)}")
+    return t.data_ptr(), (t.stride(0) if t.shape[0] > 1 else 0)
+
+
+def norm_modulate(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor] = None,
+                  shift: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None, *, kind: str = "layernorm",
+                  order: str = "norm_then_mod", eps: float = 1e-5, out: Optional[torch.Tensor] = None,
+                  out_dtype=torch.bfloat16) -> torch.Tensor:
+    """x [B, S, d] (bf16 | f32) -> y [B, S, d]; gamma/beta bf16 | f32 [d]; shift/scale f32 [1|B, d]."""
+    _dev(x, "x")
+    if x.dim() != 3:
+        raise RuntimeError("x must be [B, S, d]")
+    B, S, d = x.shape
+    _dev(gamma, "gamma")
+    if gamma.dtype not in _DT or gamma.numel() != d:
+        raise RuntimeError("gamma must be bf16 or f32 [d]")
+    if beta is not None:
+        _dev(beta, "beta", gamma.dtype)
+    sh_ptr, st1 = _rowvec(shift, "shift", d, B)
+    sc_ptr, st2 = _rowvec(scale, "scale", d, B)
+    if shift is not None and scale is not None and st1 != st2:
+        raise RuntimeError("shift and scale must share their batch stride")
+    if out is None:
+        out = torch.empty(B, S, d, dtype=out_dtype, device=x.device)
+    else:
+        _dev(out, "out")
+    L.call("aeris_norm_modulate_fwd", x.data_ptr(), _DT[x.dtype], out.data_ptr(), _DT[out.dtype], gamma.data_ptr(),
+           _ptr(beta), _DT[gamma.dtype], sh_ptr, sc_ptr, max(st1, st2), B, S, d,
+           L.NORM_LAYER if kind == "layernorm" else L.NORM_RMS,
+           L.NORM_THEN_MOD if order == "norm_then_mod" else L.MOD_THEN_NORM, float(eps), _stream())
+    return out
+
+
+_ACT = {None: L.ACT_NONE, "none": L.ACT_NONE, "gelu": L.ACT_GELU, "swiglu": L.ACT_SWIGLU, "silu": L.ACT_SILU}
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, *, act: Optional[str] = None,
+         gate: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None, rows_per_batch: int = 0,
+         out: Optional[torch.Tensor] = None, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """out[M, N] = epilogue(a[M, K] @ w[N, K]^T); see aeris_gemm_fwd in include/aeris_hip.h."""
+    _dev(a, "a", torch.bfloat16)
+    _dev(w, "w", torch.bfloat16)
+    K = a.shape[-1]
+    M = a.numel() // K
+    n_w = w.shape[0]
+    if w.shape[1] != K:
+        raise RuntimeError(f"w must be [N, {K}], got {tuple(w.shape)}")
+    N = n_w // 2 if act == "swiglu" else n_w
+    if bias is not None:
+        _dev(bias, "bias", torch.bfloat16)
+        if bias.numel() != n_w:
+            raise RuntimeError("bias has the wrong size")
+    nb = gate.shape[0] if gate is not None and gate.dim() == 2 else 1
+    if nb > 1 and (rows_per_batch <= 0 or nb * rows_per_batch != M):
+        raise RuntimeError("per-batch gate needs rows_per_batch with B * rows_per_batch == M")
+    g_ptr, gstride = _rowvec(gate, "gate", N, nb)
+    if out is None:
+        out = torch.empty(*a.shape[:-1], N, dtype=out_dtype, device=a.device)
+    else:
+        _dev(out, "out")
+        if out.numel() != M * N:
+            raise RuntimeError("out has the wrong size")
+    if residual is not None:
+        _dev(residual, "residual")
+        if residual.numel() != M * N:
+            raise RuntimeError("residual has the wrong size")
+    L.call("aeris_gemm_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), g_ptr, _ptr(residual), M, N, K,
+           N, _ACT[act], _DT[residual.dtype] if residual is not None else 0, _DT[out.dtype], gstride,
+           rows_per_batch if rows_per_batch > 0 else M, _stream())
+    return out
+
+
+def modulation_linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, *, silu: bool = False,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y f32 [B, N] = act(x f32 [B, K] @ w[N, K]^T + bias)."""
+    _dev(x, "x", torch.float32)
+    _dev(w, "w")
+    B, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K or w.dtype not in _DT:
+        raise RuntimeError("w must be bf16 or f32 [N, K]")
+    if bias is not None:
+        _dev(bias, "bias", w.dtype)
+    if out is None:
+        out = torch.empty(B, N, dtype=torch.float32, device=x.device)
+    L.call("aeris_modulation_linear_fwd", x.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), B, N, K, _DT[w.dtype],
+           L.ACT_SILU if silu else L.ACT_NONE, _stream())
+    return out
+
+
+def timestep_embedding(t: torch.Tensor, dim: int, max_period: float = 10_000.0,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(t, "t", torch.float32)
+    B = t.numel()
+    if out is None:
+        out = torch.empty(B, dim, dtype=torch.float32, device=t.device)
+    L.call("aeris_timestep_embedding_fwd", t.data_ptr(), out.data_ptr(), B, dim, float(max_period), _stream())
+    return out
+
+
+def embed_prepare(x: torch.Tensor, ape: Optional[torch.Tensor], k_pad: int, out: Optional[torch.Tensor] = None):
+    """bf16 [M, k_pad] = x f32 [M, C] (+ ape f32 [M_ape, C], row m % M_ape), zero padded."""
+    _dev(x, "x", torch.float32)
+    C = x.shape[-1]
+    M = x.numel() // C
+    m_ape = 0
+    if ape is not None:
+        _dev(ape, "ape", torch.float32)
+        m_ape = ape.numel() // C
+        if ape.shape[-1] != C or M % m_ape:
+            raise RuntimeError("ape must be [M_ape, C] with M a multiple of M_ape")
+    if out is None:
+        out = torch.empty(M, k_pad, dtype=torch.bfloat16, device=x.device)
+    L.call("aeris_embed_prepare_fwd", x.data_ptr(), _ptr(ape), out.data_ptr(), M, m_ape, C, k_pad, _stream())
+    return out

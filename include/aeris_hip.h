@@ -1,0 +1,129 @@
+/*
+ * aeris_hip.h - C ABI of libaeris_hip.so: gfx950 (MI355X) kernels for the shifted-window Swin
+ * denoiser block of AERIS window-partitioned inference.
+ *
+ * The reference has no native code and no FFI: its boundary for this path is the torch.nn.Module
+ * API of src/aeris_wp_inference/model.py.  Each entry point below replaces a sequence of
+ * ATen / einops calls of that file (cited per function).  The Python modules of the package
+ * keep the reference's class names, constructor arguments and state_dict keys and call these
+ * functions through ctypes.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and a negative AERIS_E* code on failure;
+ *     aeris_last_error() returns a thread-local description of the last failure.
+ *   - Argument validation runs on the host before anything touches the GPU, so it is testable
+ *     without a device.
+ *   - All device pointers are borrowed for the duration of the enqueue.  The library allocates
+ *     nothing, frees nothing and keeps no pointer.  Every launch is asynchronous on `stream`
+ *     (a hipStream_t passed as void*; NULL = default stream).  No hidden synchronisation,
+ *     so calls may be captured into a HIP graph.
+ *   - "bf16" = bfloat16 bits in a uint16_t; row-major everywhere; token rows are the natural
+ *     row-major lat x lon order n = Y*W + X (model.py:302).
+ */
+#ifndef AERIS_HIP_H
+#define AERIS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AERIS_OK 0
+#define AERIS_EINVAL (-1)       /* bad argument (null pointer, non-positive size, misalignment) */
+#define AERIS_EUNSUPPORTED (-2) /* shape outside what the kernels cover */
+#define AERIS_ELAUNCH (-3)      /* HIP runtime reported an error */
+
+/* element types of the tensors whose type may vary */
+#define AERIS_BF16 0
+#define AERIS_F32 1
+
+/* norm kinds / modulation order (aeris_norm_modulate_fwd) */
+#define AERIS_NORM_LAYER 0 /* (x-mean)*rsqrt(var+eps)*gamma+beta */
+#define AERIS_NORM_RMS 1   /* x*rsqrt(mean(x^2)+eps)*gamma       */
+#define AERIS_NORM_THEN_MOD 0 /* modulate(norm(x))  - model.py:426 */
+#define AERIS_MOD_THEN_NORM 1 /* norm(modulate(x))  - model.py:400-401 */
+
+/* GEMM epilogue activations (aeris_gemm_fwd) */
+#define AERIS_ACT_NONE 0
+#define AERIS_ACT_GELU 1   /* exact erf GELU */
+#define AERIS_ACT_SWIGLU 2 /* W has 2*N rows [gate | up]; C = silu(gate)*up  (model.py:156-158) */
+#define AERIS_ACT_SILU 3
+
+int aeris_version(void);
+const char* aeris_last_error(void);
+
+/* One-time per-process set-up on the current device (kernel attribute configuration).
+ * Optional: every launch entry point performs it lazily; call it before graph capture. */
+int aeris_init(void);
+
+/* ---- host-only index maps (test hooks; no GPU needed) ---------------------------------- */
+
+/* Folded partition + cyclic-roll address table.  out[(b*nWy*nWx + wy*nWx + wx)*L + iy*ws_x + ix]
+ * = b*H*W + ((wy*ws_y+iy+shift_y) mod H)*W + ((wx*ws_x+ix+shift_x) mod W).
+ * Replaces: rearrange at model.py:302/307 composed with torch.roll at model.py:111-114.
+ * This is the exact map the attention kernel uses for its loads and stores. */
+int aeris_window_index_map(int B, int H, int W, int ws_y, int ws_x, int shift_y, int shift_x,
+                           int64_t* out);
+
+/* Swin-v1 relative-position index, out[p*L+q] (no reference counterpart; textbook definition). */
+int aeris_relative_position_index(int ws_y, int ws_x, int32_t* out);
+
+/* Region id (0..8) of position (iy,ix) of window (wy,wx) on the rolled grid, out[nW*L]
+ * (the quantity the in-kernel shift mask compares; textbook Swin-v1 img_mask). */
+int aeris_shift_region_ids(int H, int W, int ws_y, int ws_x, int shift_y, int shift_x,
+                           int32_t* out);
+
+/* ---- device entry points --------------------------------------------------------------- */
+
+/* Fused windowed multi-head self-attention.
+ *   qkv  bf16 [B*H*W, 3*heads*head_dim], columns ordered (c h d): q | k | v, head-major (model.py:300)
+ *   out  bf16 [B*H*W, heads*head_dim], columns (h d) (model.py:307)
+ *   bias_table bf16 [(2ws_y-1)(2ws_x-1), heads] or NULL
+ *   use_mask != 0 adds the Swin-v1 cyclic-shift mask (-100 across regions) when a shift is non-zero
+ * Window partition / reverse and the cyclic shift are folded into the load / store addresses.
+ * Replaces model.py:300-307 (+ the swin_shift calls at model.py:471-475 on one device).
+ * Supported: ws_y*ws_x <= 256, head_dim in {32, 64}, ws_x % 4 == 0. */
+int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_table, int B, int H, int W,
+                               int heads, int head_dim, int ws_y, int ws_x, int shift_y, int shift_x,
+                               int use_mask, float scale, void* stream);
+
+/* Row norm fused with noise-level modulation.
+ *   x  [B*rows_per_batch, d] (x_dtype bf16|f32)  ->  y [B*rows_per_batch, d] (y_dtype bf16|f32)
+ *   gamma [d]; beta [d] or NULL (both param_dtype bf16|f32); shift, scale f32 [B_mod, d] or NULL
+ *   (B_mod = 1 or B, given by mod_batch_stride: 0 = one row broadcast over the batch, otherwise the
+ *   distance in elements between the rows of consecutive batch entries)
+ * Replaces torch.nn.RMSNorm + modulate (model.py:121-125,400-401,426) / LayerNorm + modulate. */
+int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,
+                            int param_dtype, const float* shift, const float* scale, int64_t mod_batch_stride,
+                            int64_t B, int64_t rows_per_batch, int d, int kind, int order, float eps,
+                            void* stream);
+
+/* C[M,N] = epilogue(A[M,K] * W[N,K]^T).
+ *   A bf16 [M,K] (lda = K); W bf16 [N,K] ([2N,K] for SWIGLU); bias bf16 [N] ([2N] for SWIGLU) or NULL
+ *   epilogue: v = acc + bias; v = act(v); if gate: v *= gate[b, n]; if residual: v += residual[m, n]
+ *   gate f32 [B_mod, N] or NULL (gate_batch_stride as above, rows_per_batch rows of C per batch entry)
+ *   residual [M, N] (res_dtype) or NULL, may alias C;  C [M, ldc] (c_dtype), ldc >= N
+ * Replaces nn.Linear at model.py:153-154,284-285,342,418 and the gate/residual elementwise passes
+ * at model.py:400-401.  Requires K % 64 == 0. */
+int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, const float* gate,
+                   const void* residual, int64_t M, int N, int K, int64_t ldc, int act, int res_dtype,
+                   int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, void* stream);
+
+/* y[b, n] = act(sum_k x[b,k] * W[n,k] + bias[n]);  x f32 [B,K], W bf16|f32 [N,K], bias same type or NULL,
+ * y f32 [B,N].  The two Linear layers of ModulationLinear (model.py:311-325) with SiLU in between. */
+int aeris_modulation_linear_fwd(const float* x, const void* W, const void* bias, float* y, int B, int N,
+                                int K, int w_dtype, int act, void* stream);
+
+/* Sinusoidal noise-level embedding [sin | cos], t f32 [B] (device) -> emb f32 [B, dim]  (model.py:127-143). */
+int aeris_timestep_embedding_fwd(const float* t, float* emb, int B, int dim, float max_period, void* stream);
+
+/* A-operand preparation for the input embedding: out bf16 [M, K_pad] = (x f32 [M, C] + ape f32 [M_ape, C] or NULL),
+ * zero padded from C to K_pad columns; ape row = m % M_ape.  (model.py:350-352) */
+int aeris_embed_prepare_fwd(const float* x, const float* ape, void* out, int64_t M, int64_t M_ape, int C,
+                            int K_pad, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AERIS_HIP_H */

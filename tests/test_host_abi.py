@@ -1,0 +1,183 @@
+"""CPU-side tests of the drop-in boundary: the C-ABI library loads, exports every symbol the header
+declares, validates arguments on the host (no GPU touched), and its index-map hooks are bit-exact
+against the oracle.  The module layer keeps the reference's state_dict layout."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+from hypothesis import given, settings, strategies as st
+
+import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    header = open(os.path.join(ROOT, "include", "aeris_hip.h")).read()
+    declared = set(re.findall(r"\b(aeris_[a-z0-9_]+)\s*\(", header))
+    assert declared, "header declares nothing?"
+    lib = pkg._lib.lib()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/aeris_hip.h but not exported"
+    assert declared == set(pkg._lib.SIGNATURES), "ctypes signature table and header disagree"
+    assert lib.aeris_version() >= 1
+
+
+CASES = [(1, 4, 8, 2, 4, 0, 0), (1, 4, 8, 2, 4, 1, 2), (2, 6, 6, 3, 2, 1, 1), (1, 32, 64, 8, 8, 4, 4),
+         (1, 180, 360, 12, 12, 6, 6), (2, 64, 96, 16, 16, 8, 8)]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_window_index_map_bit_exact(pkg, case):
+    np.testing.assert_array_equal(pkg.ops.window_index_map(*case), oracle.window_token_index(*case))
+
+
+def test_window_index_map_full_grid(pkg):
+    got = pkg.ops.window_index_map(1, 720, 1440, 16, 16, 8, 8)
+    np.testing.assert_array_equal(got, oracle.window_token_index(1, 720, 1440, 16, 16, 8, 8))
+    assert got.shape == (4050, 256)
+
+
+@settings(max_examples=30, deadline=None)
+@given(B=st.integers(1, 2), ny=st.integers(1, 4), nx=st.integers(1, 4), wy=st.integers(1, 6), wx=st.integers(1, 6), data=st.data())
+def test_window_index_map_hypothesis(pkg, B, ny, nx, wy, wx, data):
+    sy, sx = data.draw(st.integers(0, wy - 1)), data.draw(st.integers(0, wx - 1))
+    case = (B, ny * wy, nx * wx, wy, wx, sy, sx)
+    np.testing.assert_array_equal(pkg.ops.window_index_map(*case), oracle.window_token_index(*case))
+
+
+@pytest.mark.parametrize("ws", [(2, 2), (3, 5), (8, 8), (12, 12), (16, 16)])
+def test_relative_position_index_bit_exact(pkg, ws):
+    np.testing.assert_array_equal(pkg.ops.relative_position_index(*ws), oracle.relative_position_index(*ws))
+
+
+@pytest.mark.parametrize("geo", [(8, 12, 4, 4, 2, 2), (32, 64, 8, 8, 4, 4), (180, 360, 12, 12, 6, 6), (16, 16, 8, 8, 4, 0)])
+def test_shift_regions_reproduce_the_oracle_mask(pkg, geo):
+    H, W, wy, wx, sy, sx = geo
+    ids = pkg.ops.shift_region_ids(*geo)  # [nW, L]
+    mask = np.where(ids[:, :, None] != ids[:, None, :], np.float32(-100.0), np.float32(0.0))
+    np.testing.assert_array_equal(mask, oracle.shift_attention_mask(*geo))
+
+
+def test_argument_validation_needs_no_gpu(pkg):
+    L = pkg._lib
+    lib = L.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p16 = (p + 15) // 16 * 16
+    # index maps
+    assert lib.aeris_window_index_map(1, 10, 8, 4, 4, 0, 0, p) == L.EINVAL  # 10 % 4 != 0
+    assert "multiple" in L.last_error()
+    assert lib.aeris_window_index_map(1, 8, 8, 4, 4, 4, 0, p) == L.EINVAL  # shift >= window
+    assert lib.aeris_window_index_map(1, 8, 8, 4, 4, 0, 0, None) == L.EINVAL
+    assert lib.aeris_relative_position_index(0, 4, p) == L.EINVAL
+    # attention
+    f = lib.aeris_window_attention_fwd
+    assert f(None, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, None) == L.EINVAL
+    assert f(p16 + 2, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, None) == L.EINVAL  # misaligned
+    assert f(p16, p16, None, 1, 60, 60, 12, 128, 60, 60, 0, 0, 0, 0.1, None) == L.EUNSUPPORTED  # the reference's 60x60x128
+    assert "no kernel" in L.last_error()
+    assert f(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.0, None) == L.EINVAL  # scale
+    assert f(p16, p16, None, 1, 16, 20, 2, 64, 16, 16, 0, 0, 0, 0.125, None) == L.EINVAL  # grid not a multiple
+    # norm
+    g = lib.aeris_norm_modulate_fwd
+    assert g(p16, 0, p16, 0, None, None, 0, None, None, 0, 1, 4, 64, 0, 0, 1e-5, None) == L.EINVAL  # gamma NULL
+    assert g(p16, 0, p16, 0, p16, None, 0, None, None, 0, 1, 4, 60, 0, 0, 1e-5, None) == L.EUNSUPPORTED  # d % 8
+    assert g(p16, 7, p16, 0, p16, None, 0, None, None, 0, 1, 4, 64, 0, 0, 1e-5, None) == L.EINVAL  # dtype
+    assert g(p16, 0, p16, 0, p16, None, 0, None, None, 0, 1, 4, 64, 5, 0, 1e-5, None) == L.EINVAL  # kind
+    # gemm
+    h = lib.aeris_gemm_fwd
+    assert h(p16, p16, p16, None, None, None, 8, 8, 100, 8, 0, 0, 0, 0, 0, None) == L.EUNSUPPORTED  # K % 64
+    assert h(p16, p16, p16, None, None, None, 8, 8, 64, 4, 0, 0, 0, 0, 0, None) == L.EINVAL  # ldc < N
+    assert h(p16, p16, p16, None, None, None, 0, 8, 64, 8, 0, 0, 0, 0, 0, None) == L.EINVAL  # M
+    assert h(p16, p16, p16, None, None, None, 8, 8, 64, 8, 9, 0, 0, 0, 0, None) == L.EINVAL  # act
+    # small ops
+    assert lib.aeris_modulation_linear_fwd(p16, p16, None, p16, 1, 8, 12, 0, 0, None) == L.EUNSUPPORTED
+    assert lib.aeris_timestep_embedding_fwd(p16, p16, 1, 7, 10000.0, None) == L.EINVAL
+    assert lib.aeris_embed_prepare_fwd(p16, None, p16, 4, 0, 138, 128, None) == L.EINVAL  # K_pad < C
+    with pytest.raises(pkg.AerisError):
+        L.call("aeris_window_index_map", 1, 10, 8, 4, 4, 0, 0, p)
+
+
+def test_ops_refuse_cpu_tensors(pkg):
+    x = torch.zeros(1, 4, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        pkg.ops.norm_modulate(x, torch.ones(64, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="GPU"):
+        pkg.ops.gemm(x, torch.zeros(64, 64, dtype=torch.bfloat16))
+
+
+def test_ref_state_dict_layout_matches_reference(pkg):
+    """Key names, shapes and dtypes as listed for LocalAERIS (model.py:342,170,387-392,410-418,452-466)."""
+    d, heads, hd, Hd, cin, cout = 64, 2, 32, 128, 10, 5
+    m = pkg.LocalAERIS(device_mesh=None, heads=heads, dim=d, head_dim=hd, mlp_dim=Hd, window_size=(8, 8),
+                       image_shape=(16, 16), rope_base=10_000, sublayers=2, sinusoidal_emb_max_period=10_000,
+                       n_layers=4, model_in_channels=cin, model_out_channels=cout)
+    sd = m.state_dict()
+    inner = heads * hd
+    want = {"input_stage.proj.weight": ((d, cin), torch.float32), "input_stage.proj.bias": ((d,), torch.float32),
+            "input_stage.ape.inv_freq": ((3,), torch.float32),
+            "output_stage.norm.weight": ((d,), torch.float32),
+            "output_stage.modulation.0.weight": ((d, d), torch.float32), "output_stage.modulation.0.bias": ((d,), torch.float32),
+            "output_stage.modulation.2.weight": ((2 * d, d), torch.float32), "output_stage.modulation.2.bias": ((2 * d,), torch.float32),
+            "output_stage.head.weight": ((cout, d), torch.float32)}
+    for i in range(2):
+        for j in range(2):
+            p = f"layers.{i}.modulelist.{j}."
+            want.update({p + "0.weight": ((d,), torch.bfloat16), p + "1.to_qkv.weight": ((3 * inner, d), torch.bfloat16),
+                         p + "1.wo.weight": ((d, inner), torch.bfloat16), p + "2.weight": ((d,), torch.bfloat16),
+                         p + "3.w1.weight": ((2 * Hd, d), torch.bfloat16), p + "3.w2.weight": ((d, Hd), torch.bfloat16),
+                         p + "4.modulation.0.weight": ((d, d), torch.bfloat16), p + "4.modulation.0.bias": ((d,), torch.bfloat16),
+                         p + "4.modulation.2.weight": ((6 * d, d), torch.bfloat16), p + "4.modulation.2.bias": ((6 * d,), torch.bfloat16)})
+    assert set(sd.keys()) == set(want.keys())
+    for k, (shape, dt) in want.items():
+        assert tuple(sd[k].shape) == shape and sd[k].dtype == dt, k
+
+
+def test_spec_state_dict_layout(pkg):
+    layer = pkg.SwinLayer(None, 64, 2, 32, 256, (8, 8), (16, 16), True, 10_000, preset="spec", mod_ways=2)
+    keys = set(layer.state_dict().keys())
+    p = "modulelist.0."
+    assert keys == {p + k for k in ("0.weight", "0.bias", "1.to_qkv.weight", "1.to_qkv.bias", "1.wo.weight", "1.wo.bias",
+                                    "1.relative_position_bias_table", "2.weight", "2.bias", "3.fc1.weight", "3.fc1.bias",
+                                    "3.fc2.weight", "3.fc2.bias", "4.modulation.0.weight", "4.modulation.0.bias",
+                                    "4.modulation.2.weight", "4.modulation.2.bias")}
+    assert layer.state_dict()[p + "1.relative_position_bias_table"].shape == (225, 2)
+    assert layer.state_dict()[p + "4.modulation.2.weight"].shape == (4 * 64, 64)
+    assert layer.default_shift() == (4, 4)
+
+
+def test_convert_inference_checkpoint_roundtrip(pkg, tmp_path):
+    kw = dict(device_mesh=None, heads=2, dim=64, head_dim=32, mlp_dim=128, window_size=(8, 8), image_shape=(16, 16),
+              rope_base=10_000, sublayers=1, sinusoidal_emb_max_period=10_000, n_layers=4, model_in_channels=10,
+              model_out_channels=5)
+    src = pkg.LocalAERIS(**kw)
+    N = 4
+    stages = [dict() for _ in range(N)]
+    for k, v in src.state_dict().items():
+        if k.startswith("input_stage."):
+            stages[0][k[len("input_stage."):]] = v
+        elif k.startswith("output_stage."):
+            stages[N - 1][k[len("output_stage."):]] = v
+        else:
+            _, i, rest = k.split(".", 2)
+            stages[int(i) + 1][rest] = v
+    stages[0]["latent_embed.weight"] = torch.zeros(3)  # stray entries the converter must drop (model.py:483,488)
+    stages[1]["modulelist.0.1.norm.weight"] = torch.zeros(3)
+    for k, s in enumerate(stages):
+        torch.save({"ema_state_dict": s}, tmp_path / f"checkpoint_PP{k}.pth")
+    dst = pkg.LocalAERIS(**kw)
+    pkg.convert_inference_checkpoint(str(tmp_path), N, dst)
+    for k, v in src.state_dict().items():
+        assert torch.equal(dst.state_dict()[k], v), k
+    del stages[2]["modulelist.0.3.w2.weight"]
+    torch.save({"ema_state_dict": stages[2]}, tmp_path / "checkpoint_PP2.pth")
+    with pytest.raises(KeyError):
+        pkg.convert_inference_checkpoint(str(tmp_path), N, dst)
+
+
+def test_host_sigma_schedule_matches_oracle(pkg):
+    torch.testing.assert_close(pkg.sigma_schedule(10), oracle.sigma_schedule(10), rtol=0, atol=0)

@@ -18,6 +18,45 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+# Optional per-launch timing (used by bench.py): HIP events recorded on the launch stream around each kernel.
+_profile = None
+
+
+def profile_begin():
+    global _profile
+    _profile = []
+
+
+def profile_end():
+    """-> list of (tag, algorithmic work, unit, milliseconds); synchronises."""
+    global _profile
+    rec, _profile = _profile or [], None
+    torch.cuda.synchronize()
+    return [(tag, work, unit, a.elapsed_time(b)) for tag, work, unit, a, b in rec]
+
+
+class _timed:
+    def __init__(self, tag, work, unit):
+        self.on = _profile is not None
+        if self.on:
+            self.rec = [tag, work, unit, torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)]
+
+    def __enter__(self):
+        if self.on:
+            self.rec[3].record()
+
+    def __exit__(self, *exc):
+        if self.on:
+            self.rec[4].record()
+            _profile.append(tuple(self.rec))
+
+
+def gemm_uses_big_tiles(M, N, act=None):
+    """Mirror of the tile choice in csrc/gemm.hip (256x256 tiles vs 128x128), used to label timings."""
+    bn = 128 if act == "swiglu" else 256
+    return M >= 256 and (N % bn == 0 or N >= 4 * bn) and ((M + 255) // 256) * ((N + bn - 1) // bn) >= 256 and N % 4 == 0
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
@@ -83,9 +122,11 @@ def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], he
         _dev(out, "out", torch.bfloat16)
         if out.numel() != B * H * W * inner:
             raise RuntimeError("out has the wrong size")
-    L.call("aeris_window_attention_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads, head_dim,
-           window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
-           float(head_dim ** -0.5 if scale is None else scale), _stream())
+    Lw = window_size[0] * window_size[1]
+    with _timed("window_attention", 4.0 * B * H * W * Lw * inner, "flop"):
+        L.call("aeris_window_attention_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads, head_dim,
+               window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
+               float(head_dim ** -0.5 if scale is None else scale), _stream())
     return out
 
 
@@ -122,10 +163,11 @@ def norm_modulate(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Ten
         out = torch.empty(B, S, d, dtype=out_dtype, device=x.device)
     else:
         _dev(out, "out")
-    L.call("aeris_norm_modulate_fwd", x.data_ptr(), _DT[x.dtype], out.data_ptr(), _DT[out.dtype], gamma.data_ptr(),
-           _ptr(beta), _DT[gamma.dtype], sh_ptr, sc_ptr, max(st1, st2), B, S, d,
-           L.NORM_LAYER if kind == "layernorm" else L.NORM_RMS,
-           L.NORM_THEN_MOD if order == "norm_then_mod" else L.MOD_THEN_NORM, float(eps), _stream())
+    with _timed("norm_modulate", float(B * S * d * (x.element_size() + out.element_size())), "byte"):
+        L.call("aeris_norm_modulate_fwd", x.data_ptr(), _DT[x.dtype], out.data_ptr(), _DT[out.dtype], gamma.data_ptr(),
+               _ptr(beta), _DT[gamma.dtype], sh_ptr, sc_ptr, max(st1, st2), B, S, d,
+               L.NORM_LAYER if kind == "layernorm" else L.NORM_RMS,
+               L.NORM_THEN_MOD if order == "norm_then_mod" else L.MOD_THEN_NORM, float(eps), _stream())
     return out
 
 
@@ -162,9 +204,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         _dev(residual, "residual")
         if residual.numel() != M * N:
             raise RuntimeError("residual has the wrong size")
-    L.call("aeris_gemm_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), g_ptr, _ptr(residual), M, N, K,
-           N, _ACT[act], _DT[residual.dtype] if residual is not None else 0, _DT[out.dtype], gstride,
-           rows_per_batch if rows_per_batch > 0 else M, _stream())
+    tag = "gemm_256x256" if gemm_uses_big_tiles(M, N, act) else "gemm_128x128"
+    with _timed(tag, 2.0 * M * n_w * K, "flop"):
+        L.call("aeris_gemm_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), g_ptr, _ptr(residual), M, N, K,
+               N, _ACT[act], _DT[residual.dtype] if residual is not None else 0, _DT[out.dtype], gstride,
+               rows_per_batch if rows_per_batch > 0 else M, _stream())
     return out
 
 

@@ -1,0 +1,183 @@
+"""Benchmark of the hot path: one full denoiser step on the 720x1440 grid, bf16, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config1] [--no-cpu-baseline]
+
+A "step" is one denoiser forward (one function evaluation of the diffusion sampler): 138-channel input ->
+1x1 embedding to dim 1536 -> 24 Swin blocks (alternating un-shifted / half-window-shifted 16x16 windows,
+24 heads x 64, LayerNorm + per-block scale/shift from the noise-level embedding, rel-pos bias, shift mask,
+GELU MLP x4) -> linear head to 69 channels.  Random-init weights, Gaussian inputs, all resident in HBM
+before the timed region.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+WORKLOADS = {
+    # name: grid, dim, heads, head_dim, window, mlp, blocks, in/out channels
+    "config3": dict(image_shape=(720, 1440), dim=1536, heads=24, head_dim=64, window=16, mlp_dim=6144, blocks=24,
+                    cin=138, cout=69, desc="configs[3]: full denoiser step, 720x1440 grid, 24 blocks, dim 1536, 24x64 heads, 16x16 windows"),
+    "config2": dict(image_shape=(720, 1440), dim=1024, heads=16, head_dim=64, window=16, mlp_dim=4096, blocks=1,
+                    cin=138, cout=69, desc="configs[2]-shaped denoiser with ONE shifted block, dim 1024, 16x64 heads"),
+    "config1": dict(image_shape=(180, 360), dim=512, heads=8, head_dim=64, window=12, mlp_dim=2048, blocks=2,
+                    cin=138, cout=69, desc="configs[1]-shaped denoiser, 180x360 grid, 2 blocks, dim 512, 12x12 windows"),
+}
+
+
+def build_model(pkg, torch, wl, device, residual_dtype):
+    ws = wl["window"]
+    model = pkg.LocalAERIS(device_mesh=None, heads=wl["heads"], dim=wl["dim"], head_dim=wl["head_dim"],
+                           mlp_dim=wl["mlp_dim"], window_size=(ws, ws), image_shape=wl["image_shape"], rope_base=10_000,
+                           sublayers=1, sinusoidal_emb_max_period=10_000, n_layers=wl["blocks"] + 2,
+                           model_in_channels=wl["cin"], model_out_channels=wl["cout"], preset="spec", mod_ways=2,
+                           residual_dtype=residual_dtype)
+    model = model.to(device)
+    g = torch.Generator(device=device).manual_seed(0)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() >= 2:  # Linear weights and the rel-pos tables: trunc-normal(0.02); effectively un-truncated
+                p.copy_((0.02 * torch.randn(p.shape, generator=g, device=device, dtype=torch.float32)).clamp_(-2, 2).to(p.dtype))
+            elif name.endswith("bias"):
+                p.zero_()
+            else:
+                p.fill_(1.0)
+    return model
+
+
+def cpu_baseline(torch, wl, rows, seconds_cap=60.0):
+    """Time the fp32 oracle (this repository's CPU restatement of the reference block) on a strip of the same
+    grid: `rows` lat rows x full longitude, one un-shifted and one shifted block, and scale to a full step."""
+    import oracle
+    H, W = wl["image_shape"]
+    ws = wl["window"]
+    threads = torch.get_num_threads()
+    cfg = oracle.OracleConfig.spec(dim=wl["dim"], heads=wl["heads"], head_dim=wl["head_dim"], mlp_dim=wl["mlp_dim"],
+                                   window_size=(ws, ws), image_shape=(rows, W), mod_ways=2)
+    sd = oracle.init_block_weights(cfg, 0)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, rows * W, wl["dim"], generator=g)
+    t = torch.randn(1, wl["dim"], generator=g)
+    with torch.no_grad():
+        warm = oracle.OracleConfig.spec(dim=wl["dim"], heads=wl["heads"], head_dim=wl["head_dim"], mlp_dim=wl["mlp_dim"],
+                                        window_size=(ws, ws), image_shape=(ws, 4 * ws), mod_ways=2)
+        oracle.block_forward(warm, sd, x[:, :4 * ws * ws], t, (0, 0))  # warm the thread pool and the allocator
+        t0 = time.perf_counter()
+        oracle.block_forward(cfg, sd, x, t, (0, 0))
+        t_even = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        oracle.block_forward(cfg, sd, x, t, (ws // 2, ws // 2))
+        t_odd = time.perf_counter() - t0
+    scale = H / rows
+    step_s = (t_even + t_odd) / 2 * wl["blocks"] * scale  # embedding and head (1 % of the FLOPs) left out
+    return {"value": 1.0 / step_s, "unit": "denoise steps/s", "cores": threads, "kind": "port",
+            "sample": f"fp32 torch oracle, one un-shifted + one shifted block on a {rows}x{W} strip "
+                      f"({t_even:.2f}s + {t_odd:.2f}s), scaled x{scale:.1f} rows x{wl['blocks']} blocks (extrapolated)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
+    ap.add_argument("--residual", default="bf16", choices=["bf16", "f32"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=32)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the whole grid on ONE GPU; --gpus N > 1 is not supported "
+              "(no collectives, no sharding in this tier)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    pkg = importlib.import_module("aeris-gb_amd")
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    pkg._lib.call("aeris_init")
+    wl = WORKLOADS[args.workload]
+    H, W = wl["image_shape"]
+    S = H * W
+    res_dt = torch.bfloat16 if args.residual == "bf16" else torch.float32
+    model = build_model(pkg, torch, wl, dev, res_dt)
+    g = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(1, S, wl["cin"], generator=g, device=dev)
+    t = (torch.rand(1, generator=g, device=dev) * (math.pi / 2))
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            out = model(x, t)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = model(x, t)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        finite = bool(torch.isfinite(out).all())
+        # per-kernel timing with HIP events on the launch stream, over the same K steps
+        pkg.ops.profile_begin()
+        for _ in range(args.steps):
+            model(x, t)
+        rec = pkg.ops.profile_end()
+
+    ms_per_step = elapsed / args.steps * 1e3
+    agg = {}
+    for tag, work, unit, ms in rec:
+        a = agg.setdefault(tag, {"launches": 0, "work": 0.0, "ms": 0.0, "unit": unit})
+        a["launches"] += 1
+        a["work"] += work
+        a["ms"] += ms
+    kernels = {}
+    for tag, a in agg.items():
+        rate = a["work"] / (a["ms"] * 1e-3)
+        if a["unit"] == "flop":
+            kernels[tag] = {"launches_per_step": a["launches"] // args.steps, "avg_ms": a["ms"] / a["launches"],
+                            "ms_per_step": a["ms"] / args.steps, "tflops": rate / 1e12,
+                            "frac_mfma_peak": rate / 1e12 / PEAK_BF16_TFLOPS}
+        else:
+            kernels[tag] = {"launches_per_step": a["launches"] // args.steps, "avg_ms": a["ms"] / a["launches"],
+                            "ms_per_step": a["ms"] / args.steps, "gbs": rate / 1e9, "frac_hbm_peak": rate / 1e9 / PEAK_HBM_GBS}
+    if "window_attention" in kernels:  # q, k, v in + o out, bf16: 8 * S * inner bytes per launch
+        k = kernels["window_attention"]
+        byts = 8.0 * S * wl["heads"] * wl["head_dim"]
+        k["gbs"] = byts / (k["avg_ms"] * 1e-3) / 1e9
+        k["frac_hbm_peak"] = k["gbs"] / PEAK_HBM_GBS
+    dom = kernels.get("gemm_256x256")
+    roofline = None
+    if dom:
+        a = agg["gemm_256x256"]
+        roofline = {"kernel": "gemm_bf16_nt_kernel<256,256,2,4> (qkv / proj / fc1 / fc2 / embedding GEMMs)",
+                    "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": dom["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
+                    "flop_per_launch": a["work"] / a["launches"], "avg_launch_ms": dom["avg_ms"]}
+
+    result = {
+        "metric": "denoise steps/s + window-attn MFMA util, 720x1440 grid bf16, 1 GPU",
+        "value": args.steps / elapsed, "unit": "denoise steps/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": wl["desc"], "tokens": S, "batch": 1, "residual_stream": args.residual,
+                   "preset": "spec (LayerNorm, scale/shift modulation, rel-pos bias, shift mask, GELU MLP, biases)"},
+        "roofline": roofline, "kernels": kernels, "output_finite": finite,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, wl, args.cpu_rows)
+        result["gpu_over_cpu"] = result["value"] / result["cpu_baseline"]["value"]
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,148 @@
+"""GPU parity of the Swin block, the full denoiser and the sampler against the fp32 CPU oracle.
+
+Bar (from the benchmark definition): bf16 output within relative L2 <= 1e-2 of the fp32 oracle on identical
+seeded inputs; the attention-branch and MLP-branch outputs are compared as well because with the plain
+random init (std 0.02) the residual dominates the block output.
+"""
+import math
+
+import pytest
+import torch
+
+import oracle
+from oracle import OracleConfig
+from helpers import make_layer, make_model, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+CONFIG0 = dict(dim=128, heads=4, head_dim=32, mlp_dim=512, window_size=(8, 8), image_shape=(32, 64))
+CONFIG1 = dict(dim=512, heads=8, head_dim=64, mlp_dim=2048, window_size=(12, 12), image_shape=(180, 360))
+SMALL16 = dict(dim=256, heads=4, head_dim=64, mlp_dim=1024, window_size=(16, 16), image_shape=(32, 48))
+
+
+def _run_block(pkg, cuda, cfg, seed, nontrivial, shifted, x_dtype=torch.bfloat16, B=1):
+    sd = oracle.init_block_weights(cfg, seed, nontrivial=nontrivial)
+    g = torch.Generator().manual_seed(seed + 100)
+    S = cfg.image_shape[0] * cfg.image_shape[1]
+    x = torch.randn(B, S, cfg.dim, generator=g)
+    t = torch.randn(1, cfg.dim, generator=g) if cfg.mod_ways else None
+    shift = (cfg.window_size[0] // 2, cfg.window_size[1] // 2) if shifted else (0, 0)
+    xin = x.to(x_dtype)
+    ref, ref_a, ref_m = oracle.block_forward(cfg, sd, xin.float(), t, shift, return_branches=True)
+    layer = make_layer(pkg, cfg, sd, cuda, shifted)
+    br = {}
+    out = layer(xin.to(cuda), None if t is None else t.to(cuda), branches=br)
+    torch.cuda.synchronize()
+    assert out.dtype == x_dtype and out.shape == x.shape
+    return rel_l2(out, ref), rel_l2(br["attn"], ref_a), rel_l2(br["mlp"], ref_m)
+
+
+@pytest.mark.parametrize("shifted", [False, True])
+def test_config0_block(pkg, cuda, shifted):
+    """configs[0]: 32x64 grid, dim 128, 4x32 heads, 8x8 windows, shift 4, rel-pos bias, mask, LN, GELU x4."""
+    cfg = OracleConfig.spec(**CONFIG0)
+    e_out, e_attn, e_mlp = _run_block(pkg, cuda, cfg, 0, False, shifted)
+    assert e_out <= 1e-2 and e_attn <= 1e-2 and e_mlp <= 1e-2, (e_out, e_attn, e_mlp)
+
+
+@pytest.mark.parametrize("shifted", [False, True])
+def test_config1_block(pkg, cuda, shifted):
+    """configs[1]: 180x360 grid, dim 512, 8x64 heads, 12x12 windows (450 windows of 144), shift 6."""
+    cfg = OracleConfig.spec(**CONFIG1)
+    e_out, e_attn, e_mlp = _run_block(pkg, cuda, cfg, 1, False, shifted)
+    assert e_out <= 1e-2 and e_attn <= 1e-2 and e_mlp <= 1e-2, (e_out, e_attn, e_mlp)
+
+
+@pytest.mark.parametrize("geo", [CONFIG0, SMALL16], ids=["ws8", "ws16"])
+@pytest.mark.parametrize("variant", ["spec0", "spec2", "spec3", "ref", "ref_norm_then_mod", "spec_rms_swiglu"])
+def test_block_variants_nontrivial(pkg, cuda, geo, variant):
+    """Unit-gain weights, non-zero biases / gains / gates (~1): a dropped or misplaced term cannot hide."""
+    mk = {"spec0": lambda: OracleConfig.spec(mod_ways=0, **geo), "spec2": lambda: OracleConfig.spec(mod_ways=2, **geo),
+          "spec3": lambda: OracleConfig.spec(mod_ways=3, **geo), "ref": lambda: OracleConfig.ref(**geo),
+          "ref_norm_then_mod": lambda: OracleConfig.ref(mod_order="norm_then_mod", **geo),
+          "spec_rms_swiglu": lambda: OracleConfig.spec(norm="rmsnorm", mlp="swiglu", bias=False, mod_ways=3, **geo)}
+    cfg = mk[variant]()
+    for shifted in (False, True):
+        e_out, e_attn, e_mlp = _run_block(pkg, cuda, cfg, 7, True, shifted, B=2)
+        assert e_out <= 1e-2 and e_attn <= 1e-2 and e_mlp <= 1e-2, (variant, shifted, e_out, e_attn, e_mlp)
+
+
+def test_block_f32_residual_stream(pkg, cuda):
+    cfg = OracleConfig.ref(**SMALL16)
+    e_out, e_attn, e_mlp = _run_block(pkg, cuda, cfg, 3, True, True, x_dtype=torch.float32, B=2)
+    assert e_out <= 6e-3 and e_attn <= 1e-2 and e_mlp <= 1e-2, (e_out, e_attn, e_mlp)
+
+
+def test_ref_layer_does_not_shift_on_its_own(pkg, cuda):
+    """Like the reference's SwinLayer (model.py:368: shifted_grid is ignored), preset "ref" leaves the shift to the model."""
+    cfg = OracleConfig.ref(**CONFIG0)
+    sd = oracle.init_block_weights(cfg, 5, nontrivial=True)
+    layer = pkg.SwinLayer(None, cfg.dim, cfg.heads, cfg.head_dim, cfg.mlp_dim, cfg.window_size, cfg.image_shape, True, 10_000)
+    layer.load_state_dict(sd)
+    layer = layer.to(torch.bfloat16).to(cuda)
+    g = torch.Generator().manual_seed(9)
+    x, t = torch.randn(1, 2048, cfg.dim, generator=g).to(torch.bfloat16), torch.randn(1, cfg.dim, generator=g)
+    out = layer(x.to(cuda), t.to(cuda))
+    assert rel_l2(out, oracle.block_forward(cfg, sd, x.float(), t, (0, 0))) <= 1e-2
+    out_s = layer(x.to(cuda), t.to(cuda), shift=(4, 4))
+    assert rel_l2(out_s, oracle.block_forward(cfg, sd, x.float(), t, (4, 4))) <= 1e-2
+    assert rel_l2(out_s, out) > 1e-2
+
+
+MODEL_GEO = dict(dim=256, heads=4, head_dim=64, mlp_dim=1024, window_size=(16, 16), image_shape=(32, 64))
+
+
+@pytest.mark.parametrize("preset,res_dt", [("ref", torch.bfloat16), ("ref", torch.float32), ("spec", torch.bfloat16)])
+def test_small_model_parity(pkg, cuda, preset, res_dt):
+    """input stage -> 4 blocks (alternating shift) -> output stage, 138 -> 69 channels, with and without APE."""
+    mk = OracleConfig.ref if preset == "ref" else (lambda **kw: OracleConfig.spec(mod_ways=2, **kw))
+    cfg = mk(n_layers=6, in_channels=138, out_channels=69, **MODEL_GEO)
+    for nontrivial in (False, True):
+        sd = oracle.init_model_weights(cfg, 11, nontrivial=nontrivial)
+        model = make_model(pkg, cfg, sd, cuda, res_dt, preset)
+        g = torch.Generator().manual_seed(21)
+        B, S = 2, 32 * 64
+        x, dt = torch.randn(B, S, 138, generator=g), torch.tensor([0.9])
+        ref, ref_h = oracle.model_forward(cfg, sd, x, dt, return_hidden=True)
+        out, hid = model(x.to(cuda), dt.to(cuda), return_hidden=True)
+        torch.cuda.synchronize()
+        assert out.dtype == torch.float32 and out.shape == (B, S, 69)
+        assert rel_l2(hid, ref_h) <= 1e-2, (nontrivial, rel_l2(hid, ref_h))
+        assert rel_l2(out, ref) <= 1e-2, (nontrivial, rel_l2(out, ref))
+    # with the absolute positional encoding of the reference's input stage
+    ape = model.generate_ape()
+    H, W = cfg.image_shape
+    want_ape = oracle.positional_encoding_2d(138, H + 1, W)[1:].reshape(1, H * W, 138)
+    assert rel_l2(ape, want_ape) <= 1e-6
+    out = model(x.to(cuda), dt.to(cuda))
+    ref = oracle.model_forward(cfg, sd, x, dt, ape=want_ape)
+    assert rel_l2(out, ref) <= 1e-2
+
+
+def test_sampler_parity_and_graph_replay(pkg, cuda):
+    cfg = OracleConfig.ref(n_layers=4, in_channels=24, out_channels=8, dim=128, heads=2, head_dim=64, mlp_dim=256,
+                           window_size=(8, 8), image_shape=(16, 24))
+    sd = oracle.init_model_weights(cfg, 4, nontrivial=True)
+    model = make_model(pkg, cfg, sd, cuda, torch.float32, "ref")
+    g = torch.Generator().manual_seed(8)
+    B, S = 2, 16 * 24
+    cond, lat = torch.randn(B, S, 16, generator=g), torch.randn(B, S, 8, generator=g)
+    n = 4
+    ref = oracle.sample(lambda m, t: oracle.model_forward(cfg, sd, m, t), cond, lat, oracle.sigma_schedule(n))
+    smp = pkg.TrigFlowSampler(model, n_steps=n, device=cuda)
+    out = smp.sample(cond.to(cuda), lat.to(cuda))
+    torch.cuda.synchronize()
+    assert rel_l2(out, ref) <= 1e-2, rel_l2(out, ref)
+    # HIP-graph replay: several replays with eager work in between, each equal to the eager result bit for bit
+    smp.capture(cond.to(cuda), lat.to(cuda))
+    for k in range(3):
+        c2, l2 = cond.roll(k, 1).to(cuda), lat.roll(k, 1).to(cuda)
+        eager = smp.sample(c2, l2)
+        torch.cuda.synchronize()
+        replay = smp.sample_graph(c2, l2).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(eager, replay), k
+    # autoregressive rollout against the oracle's
+    states = smp.rollout(cond[..., :8].contiguous().to(cuda), 2, torch.Generator(device="cuda").manual_seed(3),
+                         extra_cond=cond[..., 8:].contiguous().to(cuda))
+    assert len(states) == 2 and all(torch.isfinite(s).all() for s in states)

@@ -1,0 +1,283 @@
+"""GPU parity tests of each HIP kernel, called through the C ABI, against the CPU oracle.
+
+Tolerances: index maps bit-exact; bf16 results within relative L2 <= 1e-2 of the fp32 oracle
+(most kernels are far tighter, each bound is written at its assert).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import OracleConfig
+from oracle.swin_oracle import attention_core
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
+def bf(t):
+    return t.to(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------------------------- GEMM
+
+GEMM_CASES = [
+    # M, N, K, act, bias, gate(batch), residual dtype, out dtype
+    (256, 256, 64, None, False, 0, None, torch.bfloat16),
+    (1000, 384, 128, None, True, 0, None, torch.bfloat16),        # ragged M, N = 3*128
+    (2048, 512, 128, "gelu", True, 0, None, torch.bfloat16),      # configs[0] fc1
+    (2048, 128, 512, None, True, 1, torch.bfloat16, torch.bfloat16),  # configs[0] fc2 + gate + residual
+    (777, 128, 192, "silu", False, 0, None, torch.float32),
+    (4096, 69, 256, None, False, 0, None, torch.float32),         # head: N = 69, scalar epilogue
+    (1300, 200, 64, None, True, 0, torch.float32, torch.float32),  # N % 128 != 0, vector epilogue
+    (66000, 1536, 512, None, True, 0, None, torch.bfloat16),      # big tiles (256x256), ragged M
+    (65536, 512, 2048, None, True, 4, torch.float32, torch.float32),  # big tiles, per-batch gate, f32 residual stream
+    (66000, 2048, 512, "gelu", True, 0, None, torch.bfloat16),
+    (3000, 256, 128, "swiglu", False, 0, None, torch.bfloat16),   # small-tile SwiGLU
+    (70000, 1024, 256, "swiglu", True, 0, None, torch.bfloat16),  # big-tile SwiGLU
+    (500, 100, 64, "swiglu", False, 0, None, torch.float32),      # SwiGLU with ragged N
+]
+
+
+@pytest.mark.parametrize("case", GEMM_CASES, ids=lambda c: f"M{c[0]}_N{c[1]}_K{c[2]}_{c[3]}")
+def test_gemm_parity(pkg, cuda, case):
+    M, N, K, act, has_bias, gate_b, res_dt, out_dt = case
+    g = torch.Generator().manual_seed(M + N + K)
+    a = bf(torch.randn(M, K, generator=g))
+    n_w = 2 * N if act == "swiglu" else N
+    w = bf(torch.randn(n_w, K, generator=g) / math.sqrt(K))
+    bias = bf(0.5 * torch.randn(n_w, generator=g)) if has_bias else None
+    gate = torch.randn(gate_b, N, generator=g) if gate_b else None
+    res = torch.randn(M, N, generator=g).to(res_dt) if res_dt is not None else None
+    # fp32 reference on the same (bf16-rounded) operands
+    ref = a.float() @ w.float().T
+    if bias is not None:
+        ref = ref + bias.float()
+    if act == "gelu":
+        ref = torch.nn.functional.gelu(ref)
+    elif act == "silu":
+        ref = torch.nn.functional.silu(ref)
+    elif act == "swiglu":
+        ref = torch.nn.functional.silu(ref[:, :N]) * ref[:, N:]
+    if gate is not None:
+        rpb = M // gate_b
+        ref = ref * gate.repeat_interleave(rpb, dim=0)
+    if res is not None:
+        ref = ref + res.float()
+    dev = lambda t: None if t is None else t.to(cuda)
+    out = pkg.ops.gemm(dev(a), dev(w), dev(bias), act=act, gate=dev(gate), residual=dev(res),
+                       rows_per_batch=(M // gate_b if gate_b else 0), out_dtype=out_dt)
+    torch.cuda.synchronize()
+    assert out.shape == (M, N) and out.dtype == out_dt
+    err = rel_l2(out, ref)
+    assert err <= (3e-3 if out_dt == torch.bfloat16 else 2e-5), err
+    assert torch.isfinite(out).all()
+
+
+def test_gemm_residual_in_place_and_deterministic(pkg, cuda):
+    g = torch.Generator().manual_seed(0)
+    a, w = bf(torch.randn(5000, 256, generator=g)).to(cuda), bf(torch.randn(384, 256, generator=g) / 16).to(cuda)
+    x = torch.randn(5000, 384, generator=g).to(cuda)
+    want = pkg.ops.gemm(a, w, residual=x, out_dtype=torch.float32)
+    y = x.clone()
+    pkg.ops.gemm(a, w, residual=y, out=y)  # C aliases the residual
+    assert torch.equal(y, want)
+    assert torch.equal(pkg.ops.gemm(a, w, residual=x, out_dtype=torch.float32), want)
+
+
+# ---------------------------------------------------------------------------------------------- attention
+
+ATTN_CASES = [
+    # B, H, W, heads, hd, ws, shift, bias, mask
+    (1, 32, 64, 4, 32, 8, 0, False, False),
+    (1, 32, 64, 4, 32, 8, 4, True, True),       # configs[0] geometry
+    (2, 16, 24, 2, 64, 8, 4, True, True),
+    (1, 36, 48, 8, 64, 12, 6, True, True),      # configs[1] window (L = 144, padded to 160)
+    (2, 24, 24, 3, 32, 12, 6, True, False),
+    (1, 48, 64, 3, 64, 16, 8, True, True),      # configs[2]/[3] window (L = 256)
+    (2, 32, 32, 2, 64, 16, 0, False, False),
+    (1, 32, 48, 2, 32, 16, 8, False, True),
+    (1, 16, 16, 1, 64, 16, 8, True, True),      # one window: every border region in it
+]
+
+
+@pytest.mark.parametrize("case", ATTN_CASES, ids=lambda c: f"B{c[0]}_{c[1]}x{c[2]}_h{c[3]}x{c[4]}_ws{c[5]}_s{c[6]}_b{int(c[7])}m{int(c[8])}")
+def test_window_attention_parity(pkg, cuda, case):
+    B, H, W, heads, hd, ws, sh, has_bias, use_mask = case
+    g = torch.Generator().manual_seed(H * W + heads)
+    inner = heads * hd
+    qkv = bf(torch.randn(B, H * W, 3 * inner, generator=g))
+    table = bf(0.7 * torch.randn((2 * ws - 1) ** 2, heads, generator=g)) if has_bias else None
+    cfg = OracleConfig(dim=inner, heads=heads, head_dim=hd, mlp_dim=inner, window_size=(ws, ws), image_shape=(H, W),
+                       rel_pos_bias=has_bias, shift_mask=use_mask)
+    ref = attention_core(cfg, qkv.float(), (sh, sh), None if table is None else table.float())
+    out = pkg.ops.window_attention(qkv.to(cuda).view(B * H * W, -1), B, (H, W), heads, hd, (ws, ws), (sh, sh),
+                                   None if table is None else table.to(cuda), use_mask)
+    torch.cuda.synchronize()
+    err = rel_l2(out.view(B, H * W, inner), ref)
+    assert err <= 6e-3, err  # P and O are rounded to bf16 once each
+    assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
+
+
+@pytest.mark.parametrize("geo", [(2, 32, 64, 8, 4), (1, 36, 60, 12, 6), (1, 48, 80, 16, 8), (1, 32, 32, 16, 0)])
+@pytest.mark.parametrize("disp", [(0, 0), (0, -1), (1, 0), (-2, 3)])
+def test_attention_index_map_bit_exact(pkg, cuda, geo, disp):
+    """q = k = 0 and a bias table that is 0 at one displacement and -30000 elsewhere make every query copy the
+    value of exactly one key, so the output must equal, bit for bit, v gathered through the oracle's
+    partition + roll map (and scattered back through it)."""
+    B, H, W, ws, sh = geo
+    heads, hd = 2, 64
+    inner = heads * hd
+    dy, dx = disp
+    g = torch.Generator().manual_seed(7)
+    v = bf(torch.randn(B * H * W, inner, generator=g))
+    qkv = torch.zeros(B * H * W, 3 * inner, dtype=torch.bfloat16)
+    qkv[:, 2 * inner:] = v
+    table = torch.full(((2 * ws - 1) ** 2, heads), -30000.0)
+    table[(dy + ws - 1) * (2 * ws - 1) + (dx + ws - 1)] = 0.0  # relative index of (query - key) = (dy, dx)
+    out = pkg.ops.window_attention(qkv.to(cuda), B, (H, W), heads, hd, (ws, ws), (sh, sh), bf(table).to(cuda), False)
+    torch.cuda.synchronize()
+    out = out.cpu()
+    idx = oracle.window_token_index(B, H, W, ws, ws, sh, sh)  # [nW, L]
+    checked = 0
+    for p in range(ws * ws):
+        ky, kx = p // ws - dy, p % ws - dx  # the key this query selects
+        if 0 <= ky < ws and 0 <= kx < ws:
+            q_rows, k_rows = idx[:, p], idx[:, ky * ws + kx]
+            assert torch.equal(out[q_rows], v[k_rows]), (p, disp)
+            checked += 1
+    assert checked >= (ws - 3) * (ws - 3)
+
+
+def test_attention_uniform_v_and_determinism_full_grid(pkg, cuda):
+    """configs[2] size (720x1440, 16 heads x 64, 16x16 windows, shift 8): uniform V per window => out = V;
+    two launches agree bit for bit; sampled windows match the oracle."""
+    B, H, W, heads, hd, ws, sh = 1, 720, 1440, 16, 64, 16, 8
+    inner = heads * hd
+    S = H * W
+    g = torch.Generator(device="cuda").manual_seed(3)
+    qkv = torch.randn(S, 3 * inner, generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    table = (0.5 * torch.randn((2 * ws - 1) ** 2, heads, generator=g, device=cuda)).to(torch.bfloat16)
+    out1 = pkg.ops.window_attention(qkv, B, (H, W), heads, hd, (ws, ws), (sh, sh), table, True)
+    out2 = pkg.ops.window_attention(qkv, B, (H, W), heads, hd, (ws, ws), (sh, sh), table, True)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, out2)
+    # sampled windows (first, a middle one, last row / last column / corner: the masked ones)
+    idx_all = oracle.window_token_index(B, H, W, ws, ws, sh, sh)
+    nWx = W // ws
+    picks = [0, 17 * nWx + 33, 44 * nWx + 5, 20 * nWx + (nWx - 1), 44 * nWx + nWx - 1]
+    ridx = torch.from_numpy(oracle.relative_position_index(ws, ws))
+    bias = table.float().cpu()[ridx.reshape(-1)].reshape(ws * ws, ws * ws, heads).permute(2, 0, 1)
+    mask_all = oracle.shift_attention_mask(H, W, ws, ws, sh, sh)
+    for w in picks:
+        rows = torch.from_numpy(idx_all[w])
+        win = qkv[rows.to(cuda)].float().cpu().reshape(ws * ws, 3, heads, hd)
+        q, k, v = (win[:, c].permute(1, 0, 2)[None] for c in range(3))
+        ref = oracle.window_attention(q, k, v, hd ** -0.5, bias, torch.from_numpy(mask_all[w])[None])
+        got = out1[rows.to(cuda)].float().cpu().reshape(ws * ws, heads, hd).permute(1, 0, 2)[None]
+        assert rel_l2(got, ref) <= 6e-3, w
+    # uniform V inside every window (value depends on the window only) => output equals V
+    win_of_token = torch.empty(S, dtype=torch.int64)
+    win_of_token[torch.from_numpy(idx_all.reshape(-1))] = torch.arange(idx_all.shape[0]).repeat_interleave(ws * ws)
+    vals = torch.randn(idx_all.shape[0], inner, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    qkv[:, 2 * inner:] = vals[win_of_token].to(cuda)
+    out = pkg.ops.window_attention(qkv, B, (H, W), heads, hd, (ws, ws), (sh, sh), table, True)
+    torch.cuda.synchronize()
+    diff = (out.float() - qkv[:, 2 * inner:].float()).abs().max().item()
+    assert diff <= 0.04, diff  # sum of bf16-rounded probabilities differs from the fp32 row sum by < 2^-8 relative
+
+
+# ---------------------------------------------------------------------------------------------- norm + modulation
+
+@pytest.mark.parametrize("d", [128, 512, 1024, 1536, 2048, 3072])
+@pytest.mark.parametrize("kind,order", [("layernorm", "norm_then_mod"), ("rmsnorm", "mod_then_norm"), ("layernorm", "mod_then_norm"), ("rmsnorm", "norm_then_mod")])
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float32])
+def test_norm_modulate_parity(pkg, cuda, d, kind, order, xdt):
+    B, S = 3, 333
+    g = torch.Generator().manual_seed(d)
+    x = (1.5 * torch.randn(B, S, d, generator=g) + 0.3).to(xdt)
+    gamma, beta = bf(1 + 0.2 * torch.randn(d, generator=g)), bf(0.2 * torch.randn(d, generator=g))
+    mods = 0.3 * torch.randn(B, 2 * d, generator=g)  # strided chunks of one wider matrix, like the block uses them
+    shift, scale = mods[:, :d], mods[:, d:]
+    eps = 1e-5 if kind == "layernorm" else float(torch.finfo(torch.float32).eps)
+    xf = x.float()
+
+    def norm(v):
+        if kind == "layernorm":
+            return oracle.layer_norm(v, gamma.float(), beta.float(), eps)
+        return oracle.rms_norm(v, gamma.float(), eps)
+
+    ref = norm(oracle.modulate(xf, shift, scale)) if order == "mod_then_norm" else oracle.modulate(norm(xf), shift, scale)
+    md = mods.to(cuda)
+    out = pkg.ops.norm_modulate(x.to(cuda), gamma.to(cuda), beta.to(cuda) if kind == "layernorm" else None,
+                                md[:, :d], md[:, d:], kind=kind, order=order, eps=eps)
+    torch.cuda.synchronize()
+    assert rel_l2(out, ref) <= 3e-3
+    out32 = pkg.ops.norm_modulate(x.to(cuda), gamma.to(cuda), beta.to(cuda) if kind == "layernorm" else None,
+                                  md[:, :d], md[:, d:], kind=kind, order=order, eps=eps, out_dtype=torch.float32)
+    assert rel_l2(out32, ref) <= 1e-5
+
+
+def test_norm_modulate_variants(pkg, cuda):
+    d, B, S = 512, 2, 50
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(B, S, d, generator=g)
+    gamma32, beta32 = 1 + 0.2 * torch.randn(d, generator=g), 0.2 * torch.randn(d, generator=g)
+    # f32 parameters, no modulation
+    out = pkg.ops.norm_modulate(x.to(cuda), gamma32.to(cuda), beta32.to(cuda), kind="layernorm", out_dtype=torch.float32)
+    assert rel_l2(out, oracle.layer_norm(x, gamma32, beta32, 1e-5)) <= 1e-5
+    # one modulation row broadcast over the batch; shift only (scale None => x + shift, model.py:122-123)
+    sh = torch.randn(1, d, generator=g)
+    out = pkg.ops.norm_modulate(x.to(cuda), gamma32.to(cuda), None, sh.to(cuda), None, kind="rmsnorm",
+                                order="mod_then_norm", eps=1e-6, out_dtype=torch.float32)
+    assert rel_l2(out, oracle.rms_norm(oracle.modulate(x, sh, None), gamma32, 1e-6)) <= 1e-5
+    # a single row, and a row count that is not a multiple of the block's 4 waves
+    x1 = torch.randn(1, 1, d, generator=g)
+    out = pkg.ops.norm_modulate(x1.to(cuda), gamma32.to(cuda), beta32.to(cuda), out_dtype=torch.float32)
+    assert rel_l2(out, oracle.layer_norm(x1, gamma32, beta32, 1e-5)) <= 1e-5
+
+
+# ---------------------------------------------------------------------------------------------- small ops
+
+@pytest.mark.parametrize("wdt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B", [1, 4, 9])
+def test_modulation_linear_parity(pkg, cuda, wdt, B):
+    d = 384
+    g = torch.Generator().manual_seed(B)
+    t = torch.randn(B, d, generator=g)
+    w0, b0 = (torch.randn(d, d, generator=g) / math.sqrt(d)).to(wdt), (0.1 * torch.randn(d, generator=g)).to(wdt)
+    w2, b2 = (torch.randn(6 * d, d, generator=g) / math.sqrt(d)).to(wdt), (0.1 * torch.randn(6 * d, generator=g)).to(wdt)
+    ref = oracle.modulation_mlp(t, w0.float(), b0.float(), w2.float(), b2.float())
+    h = pkg.ops.modulation_linear(t.to(cuda), w0.to(cuda), b0.to(cuda), silu=True)
+    out = pkg.ops.modulation_linear(h, w2.to(cuda), b2.to(cuda))
+    torch.cuda.synchronize()
+    assert rel_l2(out, ref) <= 1e-5
+
+
+def test_timestep_embedding_parity(pkg, cuda):
+    t = torch.tensor([0.0, 0.3, math.pi / 2, 1.2])
+    for dim in (128, 1536):
+        out = pkg.ops.timestep_embedding(t.to(cuda), dim, 10_000.0)
+        ref = oracle.timestep_embedding(t.double(), dim, 10_000)
+        assert (out.double().cpu() - ref).abs().max() < 2e-6
+    out0 = pkg.ops.timestep_embedding(torch.zeros(1, device=cuda), 64)
+    assert torch.equal(out0[0, :32].cpu(), torch.zeros(32)) and torch.equal(out0[0, 32:].cpu(), torch.ones(32))
+
+
+def test_embed_prepare_parity(pkg, cuda):
+    g = torch.Generator().manual_seed(2)
+    B, S, C = 2, 300, 138
+    x, ape = torch.randn(B * S, C, generator=g), torch.randn(S, C, generator=g)
+    out = pkg.ops.embed_prepare(x.to(cuda), ape.to(cuda), 192).cpu()
+    ref = torch.zeros(B * S, 192)
+    ref[:, :C] = x + ape.repeat(B, 1)
+    assert torch.equal(out, ref.to(torch.bfloat16))
+    out = pkg.ops.embed_prepare(x.to(cuda), None, 192).cpu()
+    ref[:, :C] = x
+    assert torch.equal(out, ref.to(torch.bfloat16))

@@ -12,33 +12,10 @@
 //     n fastest, which keeps the A row panels of a range in that XCD's L2
 // Epilogue (all optional, fused): + bias[n], GELU / SiLU / SwiGLU, * gate[b, n], + residual[m, n].
 #include "common.h"
+#include "gemm_common.h"
 #include "kernels.h"
 
 namespace aeris {
-
-struct GemmParams {
-  const uint16_t* A;
-  const uint16_t* W;
-  void* C;
-  const uint16_t* bias;
-  const float* gate;
-  const void* residual;
-  int64_t M;
-  int N;  // logical output columns
-  int K;
-  int64_t ldc;
-  int64_t gate_batch_stride;
-  int64_t rows_per_batch;
-  int tiles_n;
-  int act;
-  int res_dtype;  // -1 none, AERIS_BF16, AERIS_F32
-  int c_dtype;
-};
-
-__device__ __forceinline__ uint32_t swz_off(int row, int chunk) {
-  // byte offset of 16-byte chunk `chunk` (0..7) of tile row `row` in a [rows][64] bf16 tile
-  return (uint32_t)((row >> 1) * 256 + (((((row & 1) << 3) | chunk) ^ ((row >> 1) & 7)) << 4));
-}
 
 template <int BM, int BN, int WM, int WN, bool SWIGLU, bool VEC>
 __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_nt_kernel(GemmParams p) {
@@ -265,14 +242,12 @@ hipError_t gemm_configure_all() {
   e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_kernel<BM, BN, WM, WN, SG, VC>),          \
                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * (BM + BN) * 64 * 2);                 \
   if (e != hipSuccess) return e;
-  CFG(256, 256, 2, 4, false, true)
-  CFG(256, 256, 2, 4, true, true)
   CFG(128, 128, 2, 2, false, true)
   CFG(128, 128, 2, 2, true, true)
   CFG(128, 128, 2, 2, false, false)
   CFG(128, 128, 2, 2, true, false)
 #undef CFG
-  return hipSuccess;
+  return gemm_persistent_configure();
 }
 
 hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, const float* gate,
@@ -300,8 +275,10 @@ hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, 
   // vector epilogue (8 / 16 byte accesses to C and the residual) needs 4-element alignment of every row
   const bool vec = ((ldc & 3) == 0) && ((N & 3) == 0);
   if (!vec) return swiglu ? launch_gemm<128, 128, 2, 2, true, false>(p, stream) : launch_gemm<128, 128, 2, 2, false, false>(p, stream);
-  if (swiglu) return big ? launch_gemm<256, 256, 2, 4, true, true>(p, stream) : launch_gemm<128, 128, 2, 2, true, true>(p, stream);
-  return big ? launch_gemm<256, 256, 2, 4, false, true>(p, stream) : launch_gemm<128, 128, 2, 2, false, true>(p, stream);
+  // (gate rows must allow 16-byte loads: the stride between batch rows is a multiple of 4 floats)
+  const bool aligned = (reinterpret_cast<uintptr_t>(gate) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0;
+  if (big && act != AERIS_ACT_SILU && (gate_batch_stride & 3) == 0 && aligned) return gemm_persistent_launch(p, stream);
+  return swiglu ? launch_gemm<128, 128, 2, 2, true, true>(p, stream) : launch_gemm<128, 128, 2, 2, false, true>(p, stream);
 }
 
 }  // namespace aeris

@@ -1,0 +1,40 @@
+// Parameter block and LDS swizzle shared by the GEMM kernels.
+#pragma once
+#include "common.h"
+
+namespace aeris {
+
+struct GemmParams {
+  const uint16_t* A;
+  const uint16_t* W;
+  void* C;
+  const uint16_t* bias;
+  const float* gate;
+  const void* residual;
+  int64_t M;
+  int N;  // logical output columns
+  int K;
+  int64_t ldc;
+  int64_t gate_batch_stride;
+  int64_t rows_per_batch;
+  int tiles_n;
+  // persistent kernel only: tile schedule
+  int tiles_m;
+  int total_tiles;
+  int per_xcd;  // tiles in one XCD's contiguous chunk
+  int bpx;      // workgroups per XCD
+  int act;
+  int res_dtype;  // -1 none, AERIS_BF16, AERIS_F32
+  int c_dtype;
+};
+
+__device__ __forceinline__ uint32_t swz_off(int row, int chunk) {
+  // byte offset of 16-byte chunk `chunk` (0..7) of tile row `row` in a [rows][64] bf16 tile
+  return (uint32_t)((row >> 1) * 256 + (((((row & 1) << 3) | chunk) ^ ((row >> 1) & 7)) << 4));
+}
+
+// 256x256 persistent kernel (gemm_persistent.hip); needs N % 4 == 0 and ldc % 4 == 0
+hipError_t gemm_persistent_configure();
+hipError_t gemm_persistent_launch(const GemmParams& p, hipStream_t stream);
+
+}  // namespace aeris

@@ -1,0 +1,370 @@
+// Persistent bf16 MFMA GEMM for gfx950, 256x256x64 tiles:  C[M,N] = epilogue(A[M,K] * W[N,K]^T)
+//
+// Same fragment layout and LDS swizzle as the plain tile kernel (gemm.hip), restructured around the
+// two things that bound it on MI355X: the latency of the global loads of a k-tile (L2 misses of a
+// k-tile stall the whole workgroup at the barrier) and the un-overlapped prologue / epilogue of
+// every tile when only one workgroup fits a CU.
+//   - one workgroup per CU slot walks a list of tiles (persistent); the loop runs over the flat
+//     sequence (tile, k-tile), so the loads of the next tile's first k-tiles are already in flight
+//     while the epilogue of the current tile runs
+//   - global loads run one k-tile ahead of the MFMAs through registers (two LDS stages, one barrier
+//     per k-tile)
+//   - tiles are ordered so that the workgroups resident on one XCD (blockIdx % 8) cover a
+//     contiguous chunk, 4 row panels x all column tiles at a time: few distinct A / W k-slices per
+//     step compete for that XCD's 4 MB L2
+//   - the epilogue goes through a wave-private 4 KB LDS staging area: fragments (4 consecutive n per
+//     lane) are written swizzled, read back row-contiguous, and C / residual are accessed as full
+//     128-byte row segments (8 lanes x 16 B)
+#include "common.h"
+#include "gemm_common.h"
+#include "kernels.h"
+
+namespace aeris {
+
+namespace {
+constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 4;
+constexpr int NT = WM * WN * 64;          // 512 threads
+constexpr int FM = BM / WM / 32;          // 4
+constexpr int FN = BN / WN / 32;          // 2
+constexpr int A_BYTES = BM * BK * 2;      // 32 KB
+constexpr int B_BYTES = BN * BK * 2;      // 32 KB
+constexpr int STAGE = A_BYTES + B_BYTES;  // 64 KB
+constexpr int RP = NT / 8;                // 64 tile rows per loader pass
+constexpr int A_IT = BM / RP;             // 4
+constexpr int B_IT = BN / RP;             // 4
+constexpr int EPI_OFF = 2 * STAGE;        // wave-private staging, 4 KB per wave
+constexpr int SMEM = 2 * STAGE + 8 * 4096;
+constexpr int GM = 4;                     // row panels per L2 group
+}  // namespace
+
+template <int ACT, bool OUT_F32>
+__global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams p) {
+  constexpr bool SWIGLU = ACT == AERIS_ACT_SWIGLU;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int l31 = lane & 31, hi = lane >> 5;
+  const int lc = tid & 7, lr = tid >> 3;
+  const int K = p.K, N = p.N;
+  const int KT = K / BK;
+
+  // ---- this workgroup's tile list: XCD x owns tiles [x*per_xcd, (x+1)*per_xcd), slot k takes every bpx-th
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int chunk0 = xcd * p.per_xcd;
+  int chunk_len = p.total_tiles - chunk0;
+  if (chunk_len > p.per_xcd) chunk_len = p.per_xcd;
+  const int n_my = chunk_len > slot ? (chunk_len - slot + p.bpx - 1) / p.bpx : 0;
+  if (n_my == 0) return;
+
+  auto decode = [&](int r, int& tile_m, int& tile_n) {
+    const int t = chunk0 + r * p.bpx + slot;
+    const int gsz = GM * p.tiles_n;
+    const int grp = t / gsz, within = t - grp * gsz;
+    int gm = p.tiles_m - grp * GM;
+    if (gm > GM) gm = GM;
+    tile_n = within / gm;
+    tile_m = grp * GM + (within - tile_n * gm);
+  };
+
+  // ---- loader state (runs two k-tiles ahead of the compute state)
+  const uint16_t* ld_a = nullptr;
+  const uint16_t* ld_b = nullptr;
+  uint32_t a_goff[A_IT], b_goff[B_IT];
+  int ld_r = 0, ld_kt = 0;
+  auto ld_set_tile = [&]() {
+    if (ld_r >= n_my) return;
+    int tile_m, tile_n;
+    decode(ld_r, tile_m, tile_n);
+    const int64_t m0 = (int64_t)tile_m * BM;
+    const int n0 = tile_n * BN_OUT;
+    const int64_t last = p.M - 1 - m0;
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+      int64_t r = lr + i * RP;
+      if (r > last) r = last;
+      a_goff[i] = (uint32_t)(r * K + lc * 8);
+    }
+    ld_a = p.A + m0 * K;
+    int first_row = SWIGLU ? 0 : n0;
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) {
+      const int j = lr + i * RP;
+      int r;
+      if (SWIGLU) {
+        constexpr int WNW = BN / WN;  // columns of the tile owned by one wave: [gate 32 | up 32]
+        const int wv = j / WNW, within = j % WNW;
+        const int oc = n0 + wv * 32 + (within & 31);
+        r = ((within >> 5) ? N : 0) + (oc < N ? oc : N - 1);
+      } else {
+        r = n0 + j;
+        if (r > N - 1) r = N - 1;
+        r -= first_row;
+      }
+      b_goff[i] = (uint32_t)((int64_t)r * K + lc * 8);
+    }
+    ld_b = p.W + (int64_t)first_row * K;
+  };
+
+  u32x4 ra[A_IT], rb[B_IT];
+  auto issue = [&]() {
+    if (ld_r < n_my) {
+      const uint16_t* ab = ld_a + (int64_t)ld_kt * BK;
+      const uint16_t* bb = ld_b + (int64_t)ld_kt * BK;
+#pragma unroll
+      for (int i = 0; i < A_IT; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab + a_goff[i]);
+#pragma unroll
+      for (int i = 0; i < B_IT; ++i) rb[i] = *reinterpret_cast<const u32x4*>(bb + b_goff[i]);
+      if (++ld_kt == KT) {
+        ld_kt = 0;
+        ++ld_r;
+        ld_set_tile();
+      }
+    }
+  };
+  const uint32_t w_off = swz_off(lr, lc);
+  auto lstore = [&](int stage) {
+    unsigned char* s = smem + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) *reinterpret_cast<u32x4*>(s + w_off + i * RP * 128) = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) *reinterpret_cast<u32x4*>(s + A_BYTES + w_off + i * RP * 128) = rb[i];
+  };
+
+  // ---- fragment read offsets (per k16 step)
+  uint32_t a_roff[4], b_roff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    a_roff[ks] = swz_off(wm * (BM / WM) + l31, ks * 2 + hi);
+    b_roff[ks] = A_BYTES + swz_off(wn * (BN / WN) + l31, ks * 2 + hi);
+  }
+
+  f32x16 acc[FM][FN];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  };
+  zero_acc();
+
+  // ---- epilogue of the tile whose accumulators are complete
+  unsigned char* stg = smem + EPI_OFF + wave * 4096;
+  const int rrow = lane >> 3, rch = lane & 7;  // read-back mapping: row rrow + 8*it, 16-byte chunk rch
+  auto epilogue = [&](int r_done) {
+    int tile_m, tile_n;
+    decode(r_done, tile_m, tile_n);
+    const int64_t m_base = (int64_t)tile_m * BM + wm * (BM / WM);
+    const int n_wave = tile_n * BN_OUT + wn * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const int64_t m_lane = m_base + i * 32 + l31;  // row of the fragment values this lane holds
+      const float* gate_row = nullptr;
+      if (p.gate) {
+        int64_t mm = m_lane < p.M ? m_lane : p.M - 1;
+        gate_row = p.gate + (p.gate_batch_stride ? (mm / p.rows_per_batch) * p.gate_batch_stride : 0);
+      }
+      // stage 1: bias / activation / gate on one 32 x 32 fragment, 4 consecutive n per g (N % 4 == 0, so a
+      // group of 4 is entirely inside or entirely outside the matrix)
+      auto fragment = [&](int j, float (&v)[4][4]) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          int n = n_wave + j * 32 + g * 8 + hi * 4;
+          if (n >= N) n = N - 4;  // clamped group: computed but never stored
+          f32x4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f}, gt = {1.f, 1.f, 1.f, 1.f};
+          if (p.bias) {
+            const u32x2 r = *reinterpret_cast<const u32x2*>(p.bias + n);
+            b0 = f32x4{bf16_lo(r.x), bf16_hi(r.x), bf16_lo(r.y), bf16_hi(r.y)};
+            if (SWIGLU) {
+              const u32x2 r1 = *reinterpret_cast<const u32x2*>(p.bias + N + n);
+              b1 = f32x4{bf16_lo(r1.x), bf16_hi(r1.x), bf16_lo(r1.y), bf16_hi(r1.y)};
+            }
+          }
+          if (gate_row) gt = *reinterpret_cast<const f32x4*>(gate_row + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x = acc[i][j][g * 4 + e] + b0[e];
+            if (SWIGLU) x = silu_f(x) * (acc[i][1][g * 4 + e] + b1[e]);
+            else if (ACT == AERIS_ACT_GELU) x = gelu_erf_f(x);
+            v[g][e] = x * gt[e];
+          }
+        }
+      };
+      if (!OUT_F32) {
+        // stage 2 (bf16 C): whole 32 x 64 (SwiGLU: 32 x 32) block through LDS, rows of 128 B, chunk-swizzled
+#pragma unroll
+        for (int j = 0; j < (SWIGLU ? 1 : FN); ++j) {
+          float v[4][4];
+          fragment(j, v);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            u32x2 w2 = {pack_bf16x2(v[g][0], v[g][1]), pack_bf16x2(v[g][2], v[g][3])};
+            *reinterpret_cast<u32x2*>(stg + l31 * 128 + (((j * 4 + g) ^ (l31 & 7)) << 4) + hi * 8) = w2;
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int CHUNKS = SWIGLU ? 4 : 8;  // 16-byte chunks (8 columns) per staged row
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int row = rrow + 8 * it;
+          const int64_t m = m_base + i * 32 + row;
+          const int n = n_wave + rch * 8;
+          if (rch < CHUNKS && m < p.M && n < N) {
+            const u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+            const int64_t off = m * p.ldc + n;
+            const bool full = n + 8 <= N;  // N % 4 == 0: a chunk is whole or exactly half inside
+            uint16_t* cp = reinterpret_cast<uint16_t*>(p.C) + off;
+            if (p.res_dtype < 0) {
+              if (full) *reinterpret_cast<u32x4*>(cp) = w4;
+              else *reinterpret_cast<u32x2*>(cp) = u32x2{w4.x, w4.y};
+            } else {
+              float o[8];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) { o[2 * e] = bf16_lo(w4[e]); o[2 * e + 1] = bf16_hi(w4[e]); }
+              if (p.res_dtype == AERIS_BF16) {
+                const uint16_t* rp = reinterpret_cast<const uint16_t*>(p.residual) + off;
+                if (full) {
+                  const u32x4 r4 = *reinterpret_cast<const u32x4*>(rp);
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) { o[2 * e] += bf16_lo(r4[e]); o[2 * e + 1] += bf16_hi(r4[e]); }
+                } else {
+                  const u32x2 r2 = *reinterpret_cast<const u32x2*>(rp);
+                  o[0] += bf16_lo(r2.x); o[1] += bf16_hi(r2.x); o[2] += bf16_lo(r2.y); o[3] += bf16_hi(r2.y);
+                }
+              } else {
+                const float* rp = reinterpret_cast<const float*>(p.residual) + off;
+                const f32x4 r0 = *reinterpret_cast<const f32x4*>(rp);
+                o[0] += r0.x; o[1] += r0.y; o[2] += r0.z; o[3] += r0.w;
+                if (full) {
+                  const f32x4 r1 = *reinterpret_cast<const f32x4*>(rp + 4);
+                  o[4] += r1.x; o[5] += r1.y; o[6] += r1.z; o[7] += r1.w;
+                }
+              }
+              if (full) {
+                u32x4 c4 = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
+                *reinterpret_cast<u32x4*>(cp) = c4;
+              } else {
+                u32x2 c2 = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+                *reinterpret_cast<u32x2*>(cp) = c2;
+              }
+            }
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      } else {
+        // stage 2 (f32 C): 32 x 32 block per fragment column j, rows of 128 B (32 floats)
+#pragma unroll
+        for (int j = 0; j < (SWIGLU ? 1 : FN); ++j) {
+          float v[4][4];
+          fragment(j, v);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f32x4 w4 = {v[g][0], v[g][1], v[g][2], v[g][3]};
+            *reinterpret_cast<f32x4*>(stg + l31 * 128 + (((g * 2 + hi) ^ (l31 & 7)) << 4)) = w4;
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int row = rrow + 8 * it;
+            const int64_t m = m_base + i * 32 + row;
+            const int n = n_wave + j * 32 + rch * 4;
+            if (m < p.M && n < N) {
+              f32x4 o = *reinterpret_cast<const f32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+              const int64_t off = m * p.ldc + n;
+              if (p.res_dtype == AERIS_BF16) {
+                const u32x2 r2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
+                o.x += bf16_lo(r2.x); o.y += bf16_hi(r2.x); o.z += bf16_lo(r2.y); o.w += bf16_hi(r2.y);
+              } else if (p.res_dtype == AERIS_F32) {
+                const f32x4 r4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.residual) + off);
+                o.x += r4.x; o.y += r4.y; o.z += r4.z; o.w += r4.w;
+              }
+              *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + off) = o;
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+  };
+
+  // ---- flat pipeline over (tile, k-tile): loads of step j+1 are in flight while step j is computed
+  const int total = n_my * KT;
+  int c_r = 0, c_kt = 0;  // compute state
+  ld_set_tile();
+  issue();
+  lstore(0);
+  __syncthreads();
+
+  for (int j = 0; j < total; ++j) {
+    issue();
+    const unsigned char* s = smem + (j & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      bf16x8 af[FM], bfr[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(s + a_roff[ks] + i * 32 * 128);
+#pragma unroll
+      for (int jn = 0; jn < FN; ++jn) bfr[jn] = *reinterpret_cast<const bf16x8*>(s + b_roff[ks] + jn * 32 * 128);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int jn = 0; jn < FN; ++jn)
+          acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[jn], af[i], acc[i][jn], 0, 0, 0);
+    }
+    if (j + 1 < total) lstore((j + 1) & 1);
+    __syncthreads();
+    if (++c_kt == KT) {
+      epilogue(c_r);
+      zero_acc();
+      c_kt = 0;
+      ++c_r;
+    }
+  }
+}
+
+hipError_t gemm_persistent_configure() {
+  hipError_t e;
+#define CFG(A, F32)                                                                                        \
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_persistent_kernel<A, F32>),             \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);                                 \
+  if (e != hipSuccess) return e;
+  CFG(AERIS_ACT_NONE, false) CFG(AERIS_ACT_NONE, true) CFG(AERIS_ACT_GELU, false) CFG(AERIS_ACT_GELU, true)
+  CFG(AERIS_ACT_SWIGLU, false) CFG(AERIS_ACT_SWIGLU, true)
+#undef CFG
+  return hipSuccess;
+}
+
+// p.act must be NONE, GELU or SWIGLU; N % 4 == 0 and ldc % 4 == 0; bias / gate rows 8- / 16-byte aligned
+hipError_t gemm_persistent_launch(const GemmParams& p0, hipStream_t stream) {
+  GemmParams p = p0;
+  const bool swiglu = p.act == AERIS_ACT_SWIGLU;
+  const int bn_out = swiglu ? BN / 2 : BN;
+  p.tiles_m = (int)((p.M + BM - 1) / BM);
+  p.tiles_n = (p.N + bn_out - 1) / bn_out;
+  p.total_tiles = p.tiles_m * p.tiles_n;
+  p.per_xcd = (p.total_tiles + 7) / 8;
+  p.bpx = p.per_xcd < 32 ? p.per_xcd : 32;  // 32 CUs per XCD, one workgroup each
+  dim3 grid(8 * p.bpx), block(NT);
+  const bool f32 = p.c_dtype == AERIS_F32;
+#define GO(A)                                                                                              \
+  do {                                                                                                     \
+    if (f32) hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, true>), grid, block, SMEM, stream, p);    \
+    else hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, false>), grid, block, SMEM, stream, p);       \
+  } while (0)
+  if (swiglu) GO(AERIS_ACT_SWIGLU);
+  else if (p.act == AERIS_ACT_GELU) GO(AERIS_ACT_GELU);
+  else GO(AERIS_ACT_NONE);
+#undef GO
+  return hipGetLastError();
+}
+
+}  // namespace aeris

@@ -17,15 +17,14 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as
 __device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
 
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
-}
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+// round-to-nearest-even conversions; on gfx950 a pair is one v_cvt_pk_bf16_f32
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
 
 // 64-lane wavefront reductions
 __device__ __forceinline__ float wave_sum(float v) {

@@ -159,65 +159,22 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     decode(r_done, tile_m, tile_n);
     const int64_t m_base = (int64_t)tile_m * BM + wm * (BM / WM);
     const int n_wave = tile_n * BN_OUT + wn * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
-    constexpr int FNO = SWIGLU ? 1 : FN;
-
-    auto wave_sync = [&]() {  // orders this wave's LDS traffic on its private staging area
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    };
-
-    // finished values live in plain scalar registers (not in the MFMA accumulator tuples)
-    float of[OUT_F32 ? FNO : 1][16];  // f32 C: one 32-row block at a time
-    uint32_t ob[OUT_F32 ? 1 : FM][OUT_F32 ? 1 : FNO][8];
-
-    // phase A: bias / activation / gate / residual applied to the accumulators.  A lane holds 4 consecutive
-    // n per (j, g); N % 4 == 0, so such a group is entirely inside or entirely outside the matrix.  The
-    // residual is fetched as full 128-byte row segments and redistributed to the fragment layout through the
-    // staging area.  Every load of the tile happens in this phase, before its first store: the memory
-    // counter retires in order, so a load issued after a store would wait for that store's acknowledgement.
-    auto phaseA = [&](int i) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
       const int64_t m_lane = m_base + i * 32 + l31;  // row of the fragment values this lane holds
       const float* gate_row = nullptr;
       if (p.gate) {
         int64_t mm = m_lane < p.M ? m_lane : p.M - 1;
         gate_row = p.gate + (p.gate_batch_stride ? (mm / p.rows_per_batch) * p.gate_batch_stride : 0);
       }
-      if (p.res_dtype == AERIS_BF16) {  // 32 rows x 64 (SwiGLU: 32) columns, 128 B per staged row
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-          const int row = rrow + 8 * it;
-          const int64_t m = m_base + i * 32 + row;
-          const int n = n_wave + rch * 8;
-          u32x4 r = {0u, 0u, 0u, 0u};
-          if (rch < (SWIGLU ? 4 : 8) && m < p.M && n < N) {
-            const uint16_t* rp = reinterpret_cast<const uint16_t*>(p.residual) + m * p.ldc + n;
-            if (n + 8 <= N) r = *reinterpret_cast<const u32x4*>(rp);
-            else { const u32x2 t = *reinterpret_cast<const u32x2*>(rp); r.x = t.x; r.y = t.y; }
-          }
-          *reinterpret_cast<u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4)) = r;
-        }
-        wave_sync();
-      }
-#pragma unroll
-      for (int j = 0; j < FNO; ++j) {
-        if (p.res_dtype == AERIS_F32) {  // 32 rows x 32 columns of floats, 128 B per staged row
-#pragma unroll
-          for (int it = 0; it < 4; ++it) {
-            const int row = rrow + 8 * it;
-            const int64_t m = m_base + i * 32 + row;
-            const int n = n_wave + j * 32 + rch * 4;
-            u32x4 r = {0u, 0u, 0u, 0u};
-            if (m < p.M && n < N) r = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.residual) + m * p.ldc + n);
-            *reinterpret_cast<u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4)) = r;
-          }
-          wave_sync();
-        }
+      // stage 1: bias / activation / gate on one 32 x 32 fragment, 4 consecutive n per g (N % 4 == 0, so a
+      // group of 4 is entirely inside or entirely outside the matrix)
+      auto fragment = [&](int j, float (&v)[4][4]) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           int n = n_wave + j * 32 + g * 8 + hi * 4;
           if (n >= N) n = N - 4;  // clamped group: computed but never stored
-          f32x4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f}, gt = {1.f, 1.f, 1.f, 1.f}, rs = {0.f, 0.f, 0.f, 0.f};
+          f32x4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f}, gt = {1.f, 1.f, 1.f, 1.f};
           if (p.bias) {
             const u32x2 r = *reinterpret_cast<const u32x2*>(p.bias + n);
             b0 = f32x4{bf16_lo(r.x), bf16_hi(r.x), bf16_lo(r.y), bf16_hi(r.y)};
@@ -227,86 +184,115 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
             }
           }
           if (gate_row) gt = *reinterpret_cast<const f32x4*>(gate_row + n);
-          if (p.res_dtype == AERIS_BF16) {
-            const u32x2 r = *reinterpret_cast<const u32x2*>(stg + l31 * 128 + (((j * 4 + g) ^ (l31 & 7)) << 4) + hi * 8);
-            rs = f32x4{bf16_lo(r.x), bf16_hi(r.x), bf16_lo(r.y), bf16_hi(r.y)};
-          } else if (p.res_dtype == AERIS_F32) {
-            rs = *reinterpret_cast<const f32x4*>(stg + l31 * 128 + (((g * 2 + hi) ^ (l31 & 7)) << 4));
-          }
-          float x[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            x[e] = acc[i][j][g * 4 + e] + b0[e];
-            if (SWIGLU) x[e] = silu_f(x[e]) * (acc[i][1][g * 4 + e] + b1[e]);
-            else if (ACT == AERIS_ACT_GELU) x[e] = gelu_erf_f(x[e]);
-            x[e] = fmaf(x[e], gt[e], rs[e]);
-          }
-          if (OUT_F32) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) of[j][g * 4 + e] = x[e];
-          } else {
-            ob[i][j][g * 2] = pack_bf16x2(x[0], x[1]);
-            ob[i][j][g * 2 + 1] = pack_bf16x2(x[2], x[3]);
+            float x = acc[i][j][g * 4 + e] + b0[e];
+            if (SWIGLU) x = silu_f(x) * (acc[i][1][g * 4 + e] + b1[e]);
+            else if (ACT == AERIS_ACT_GELU) x = gelu_erf_f(x);
+            v[g][e] = x * gt[e];
           }
         }
-        if (p.res_dtype == AERIS_F32) wave_sync();
-      }
-      if (p.res_dtype == AERIS_BF16) wave_sync();
-    };
-
-    // phase B: fragments -> staging area -> full 128-byte row segments of C (stores only)
-    constexpr int CPL = OUT_F32 ? 4 : 8;  // output columns per lane
-    constexpr int CHUNKS = OUT_F32 ? 8 : (SWIGLU ? 4 : 8);
-    auto phaseB = [&](int i, int j0) {  // bf16 C: 32 x 64 block (j0 = 0); f32 C: one 32 x 32 fragment
-      if (OUT_F32) {
+      };
+      if (!OUT_F32) {
+        // stage 2 (bf16 C): whole 32 x 64 (SwiGLU: 32 x 32) block through LDS, rows of 128 B, chunk-swizzled
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          f32x4 w4 = {of[j0][g * 4], of[j0][g * 4 + 1], of[j0][g * 4 + 2], of[j0][g * 4 + 3]};
-          *reinterpret_cast<f32x4*>(stg + l31 * 128 + (((g * 2 + hi) ^ (l31 & 7)) << 4)) = w4;
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < FNO; ++j)
+        for (int j = 0; j < (SWIGLU ? 1 : FN); ++j) {
+          float v[4][4];
+          fragment(j, v);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            u32x2 w2 = {ob[i][j][g * 2], ob[i][j][g * 2 + 1]};
+            u32x2 w2 = {pack_bf16x2(v[g][0], v[g][1]), pack_bf16x2(v[g][2], v[g][3])};
             *reinterpret_cast<u32x2*>(stg + l31 * 128 + (((j * 4 + g) ^ (l31 & 7)) << 4) + hi * 8) = w2;
           }
-      }
-      wave_sync();
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int CHUNKS = SWIGLU ? 4 : 8;  // 16-byte chunks (8 columns) per staged row
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int row = rrow + 8 * it;
-        const int64_t m = m_base + i * 32 + row;
-        const int n = n_wave + j0 * 32 + rch * CPL;
-        if (rch < CHUNKS && m < p.M && n < N) {
-          const u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
-          const int64_t off = m * p.ldc + n;
-          if (OUT_F32) {
-            *reinterpret_cast<u32x4*>(reinterpret_cast<float*>(p.C) + off) = w4;
-          } else {
+        for (int it = 0; it < 4; ++it) {
+          const int row = rrow + 8 * it;
+          const int64_t m = m_base + i * 32 + row;
+          const int n = n_wave + rch * 8;
+          if (rch < CHUNKS && m < p.M && n < N) {
+            const u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+            const int64_t off = m * p.ldc + n;
+            const bool full = n + 8 <= N;  // N % 4 == 0: a chunk is whole or exactly half inside
             uint16_t* cp = reinterpret_cast<uint16_t*>(p.C) + off;
-            if (n + 8 <= N) *reinterpret_cast<u32x4*>(cp) = w4;
-            else *reinterpret_cast<u32x2*>(cp) = u32x2{w4.x, w4.y};
+            if (p.res_dtype < 0) {
+              if (full) *reinterpret_cast<u32x4*>(cp) = w4;
+              else *reinterpret_cast<u32x2*>(cp) = u32x2{w4.x, w4.y};
+            } else {
+              float o[8];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) { o[2 * e] = bf16_lo(w4[e]); o[2 * e + 1] = bf16_hi(w4[e]); }
+              if (p.res_dtype == AERIS_BF16) {
+                const uint16_t* rp = reinterpret_cast<const uint16_t*>(p.residual) + off;
+                if (full) {
+                  const u32x4 r4 = *reinterpret_cast<const u32x4*>(rp);
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) { o[2 * e] += bf16_lo(r4[e]); o[2 * e + 1] += bf16_hi(r4[e]); }
+                } else {
+                  const u32x2 r2 = *reinterpret_cast<const u32x2*>(rp);
+                  o[0] += bf16_lo(r2.x); o[1] += bf16_hi(r2.x); o[2] += bf16_lo(r2.y); o[3] += bf16_hi(r2.y);
+                }
+              } else {
+                const float* rp = reinterpret_cast<const float*>(p.residual) + off;
+                const f32x4 r0 = *reinterpret_cast<const f32x4*>(rp);
+                o[0] += r0.x; o[1] += r0.y; o[2] += r0.z; o[3] += r0.w;
+                if (full) {
+                  const f32x4 r1 = *reinterpret_cast<const f32x4*>(rp + 4);
+                  o[4] += r1.x; o[5] += r1.y; o[6] += r1.z; o[7] += r1.w;
+                }
+              }
+              if (full) {
+                u32x4 c4 = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
+                *reinterpret_cast<u32x4*>(cp) = c4;
+              } else {
+                u32x2 c2 = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+                *reinterpret_cast<u32x2*>(cp) = c2;
+              }
+            }
           }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      } else {
+        // stage 2 (f32 C): 32 x 32 block per fragment column j, rows of 128 B (32 floats)
+#pragma unroll
+        for (int j = 0; j < (SWIGLU ? 1 : FN); ++j) {
+          float v[4][4];
+          fragment(j, v);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f32x4 w4 = {v[g][0], v[g][1], v[g][2], v[g][3]};
+            *reinterpret_cast<f32x4*>(stg + l31 * 128 + (((g * 2 + hi) ^ (l31 & 7)) << 4)) = w4;
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int row = rrow + 8 * it;
+            const int64_t m = m_base + i * 32 + row;
+            const int n = n_wave + j * 32 + rch * 4;
+            if (m < p.M && n < N) {
+              f32x4 o = *reinterpret_cast<const f32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+              const int64_t off = m * p.ldc + n;
+              if (p.res_dtype == AERIS_BF16) {
+                const u32x2 r2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
+                o.x += bf16_lo(r2.x); o.y += bf16_hi(r2.x); o.z += bf16_lo(r2.y); o.w += bf16_hi(r2.y);
+              } else if (p.res_dtype == AERIS_F32) {
+                const f32x4 r4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.residual) + off);
+                o.x += r4.x; o.y += r4.y; o.z += r4.z; o.w += r4.w;
+              }
+              *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + off) = o;
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+        }
       }
-      wave_sync();
-    };
-
-    if (OUT_F32) {
-      // 128 finished floats per lane do not fit next to the accumulators: finish and store 32 rows at a time
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        phaseA(i);
-#pragma unroll
-        for (int j = 0; j < FNO; ++j) phaseB(i, j);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < FM; ++i) phaseA(i);
-#pragma unroll
-      for (int i = 0; i < FM; ++i) phaseB(i, 0);
     }
   };
 

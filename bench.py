@@ -155,11 +155,16 @@ def main():
         byts = 8.0 * S * wl["heads"] * wl["head_dim"]
         k["gbs"] = byts / (k["avg_ms"] * 1e-3) / 1e9
         k["frac_hbm_peak"] = k["gbs"] / PEAK_HBM_GBS
-    dom = kernels.get("gemm_256x256")
+    NAMES = {"gemm_256x256_none_bf16": "gemm_bf16_nt_persistent_kernel<0, false> (qkv / proj / fc2 / embedding GEMMs)",
+             "gemm_256x256_gelu_bf16": "gemm_bf16_nt_persistent_kernel<1, false> (fc1 GEMM + GELU)",
+             "gemm_256x256_none_f32": "gemm_bf16_nt_persistent_kernel<0, true>",
+             "gemm_256x256_swiglu_bf16": "gemm_bf16_nt_persistent_kernel<2, false>"}
+    big = [t for t in kernels if t.startswith("gemm_256x256")]
     roofline = None
-    if dom:
-        a = agg["gemm_256x256"]
-        roofline = {"kernel": "gemm_bf16_nt_kernel<256,256,2,4> (qkv / proj / fc1 / fc2 / embedding GEMMs)",
+    if big:
+        dom_tag = max(big, key=lambda t: kernels[t]["ms_per_step"])  # the kernel the step spends most time in
+        dom, a = kernels[dom_tag], agg[dom_tag]
+        roofline = {"kernel": NAMES.get(dom_tag, dom_tag),
                     "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": dom["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
                     "flop_per_launch": a["work"] / a["launches"], "avg_launch_ms": dom["avg_ms"]}

@@ -7,8 +7,9 @@
 //   - one workgroup per CU slot walks a list of tiles (persistent); the loop runs over the flat
 //     sequence (tile, k-tile), so the loads of the next tile's first k-tiles are already in flight
 //     while the epilogue of the current tile runs
-//   - global loads run one k-tile ahead of the MFMAs through registers (two LDS stages, one barrier
-//     per k-tile)
+//   - global loads of k-tile j+2 are issued in the middle of step j, right after the staging registers
+//     have been drained into the idle LDS stage (k-tile j+1): a load has a full step to arrive (two LDS
+//     stages, one barrier per k-tile)
 //   - tiles are ordered so that the workgroups resident on one XCD (blockIdx % 8) cover a
 //     contiguous chunk, 4 row panels x all column tiles at a time: few distinct A / W k-slices per
 //     step compete for that XCD's 4 MB L2
@@ -188,7 +189,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           for (int e = 0; e < 4; ++e) {
             float x = acc[i][j][g * 4 + e] + b0[e];
             if (SWIGLU) x = silu_f(x) * (acc[i][1][g * 4 + e] + b1[e]);
-            else if (ACT == AERIS_ACT_GELU) x = gelu_erf_f(x);
+            else if (ACT == AERIS_ACT_GELU) x = OUT_F32 ? gelu_erf_f(x) : gelu_bf16_f(x);
             v[g][e] = x * gt[e];
           }
         }
@@ -296,22 +297,26 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     }
   };
 
-  // ---- flat pipeline over (tile, k-tile): loads of step j+1 are in flight while step j is computed
+  // ---- flat pipeline over (tile, k-tile): a k-tile is loaded a full step before it is moved to LDS
   const int total = n_my * KT;
   int c_r = 0, c_kt = 0;  // compute state
   ld_set_tile();
   issue();
   lstore(0);
+  issue();  // k-tile 1 stays in registers until the middle of step 0
   __syncthreads();
 
   for (int j = 0; j < total; ++j) {
-    issue();
     const unsigned char* s = smem + (j & 1) * STAGE;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      // the other LDS stage is idle during this step: fill it half way through, so that the wait for the
-      // global loads overlaps with the MFMAs of the second wave on this SIMD
-      if (ks == 2 && j + 1 < total) lstore((j + 1) & 1);
+      // the other LDS stage is idle during this step: half way through, move k-tile j+1 (loaded a full step
+      // ago) from the staging registers into it and immediately reuse the registers for the loads of k-tile
+      // j+2.  The wait for the loads overlaps with the MFMAs of the second wave on this SIMD.
+      if (ks == 2 && j + 1 < total) {
+        lstore((j + 1) & 1);
+        issue();
+      }
       bf16x8 af[FM], bfr[FN];
 #pragma unroll
       for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(s + a_roff[ks] + i * 32 * 128);

@@ -5,10 +5,12 @@
 // (wy, wx) is row  b*H*W + ((wy*WS_Y + iy + sy) mod H)*W + ((wx*WS_X + ix + sx) mod W)  of the
 // natural-order qkv / out matrices, for loads and for stores alike.
 //
-// Data flow per workgroup (NW waves, wave w owns queries 32w .. 32w+31):
-//   K  [L][HD]   global -> LDS rows padded by 16 B (bank-conflict-free ds_read_b128 fragments)
+// Data flow per workgroup (ceil(NQ/2) waves; wave w processes the 32-query groups w and w + NWAVES one after
+// the other, so that a workgroup is small enough for two of them to share a CU: while one loads its K / V,
+// the other computes):
+//   K  [L][HD]   global -> LDS, 16-byte chunks XOR-swizzled (bank-conflict-free ds_read_b128 fragments)
 //   V  [L][HD]   global -> registers (4 keys x 8 d per thread) -> 4x8 register transpose ->
-//                LDS as V^T [HD][LPAD] so that PV fragments are key-contiguous ds_read_b64
+//                LDS as V^T [HD][LPAD], key groups permuted so that a PV fragment is one ds_read_b128
 //   bias table   column of this head -> LDS as fp32 4-vectors R4[s] = (R[s..s+3]), R reversed and
 //                pre-multiplied by log2(e): the biases of 4 consecutive keys are one ds_read_b128
 //   Q            global -> registers (MFMA B operand), never in LDS
@@ -37,25 +39,36 @@ struct AttnParams {
 template <int WS_Y, int WS_X, int HD, bool HAS_BIAS>
 struct AttnCfg {
   static constexpr int L = WS_Y * WS_X;
-  static constexpr int NW = (L + 31) / 32;
-  static constexpr int LPAD = NW * 32;
-  static constexpr int NT = NW * 64;
-  static constexpr int KROW = HD * 2 + 16;    // bytes
-  static constexpr int VROW = LPAD * 2 + 8;   // bytes
+  static constexpr int NQ = (L + 31) / 32;     // 32-query groups (= 32-key blocks)
+  static constexpr int LPAD = NQ * 32;
+  static constexpr int NWAVES = (NQ + 1) / 2;  // a wave processes query groups w and w + NWAVES in turn
+  static constexpr int NT = NWAVES * 64;
+  // V^T rows: XOR-swizzled 16-byte chunks when a row holds a multiple of 16 chunks, otherwise padded by 16 B
+  static constexpr bool V_SWZ = (LPAD * 2 / 16) % 16 == 0;
+  static constexpr int VROW = V_SWZ ? LPAD * 2 : LPAD * 2 + 16;  // bytes
   static constexpr int TBL = (2 * WS_Y - 1) * (2 * WS_X - 1);
-  static constexpr int K_BYTES = LPAD * KROW;
+  // K rows: 128 B chunk-swizzled (head_dim 64) or 64 B padded to 80 B (head_dim 32)
+  static constexpr int K_BYTES = HD == 64 ? LPAD * 128 : LPAD * 80;
   static constexpr int V_BYTES = ((HD * VROW + 15) / 16) * 16;
   static constexpr int B_BYTES = HAS_BIAS ? TBL * 16 : 0;
-  static constexpr int SMEM = K_BYTES + V_BYTES + B_BYTES;
+  static constexpr int SMEM = K_BYTES + V_BYTES + B_BYTES;  // 16x16 x 64 with bias: 80 912 B, two workgroups per CU
 };
 
-constexpr int attn_threads(int ws_y, int ws_x) { return ((ws_y * ws_x + 31) / 32) * 64; }
+constexpr int attn_threads(int ws_y, int ws_x) { return (((ws_y * ws_x + 31) / 32 + 1) / 2) * 64; }
+
+// byte offset of 16-byte chunk `chunk` of key row `key` in the K tile
+template <int HD>
+__device__ __forceinline__ uint32_t k_off(int key, int chunk) {
+  if (HD == 64) return (uint32_t)((key >> 1) * 256 + (((((key & 1) << 3) | chunk) ^ ((key >> 1) & 7)) << 4));
+  return (uint32_t)(key * 80 + chunk * 16);
+}
 
 template <int WS_Y, int WS_X, int HD, bool HAS_BIAS>
-__global__ void __launch_bounds__(attn_threads(WS_Y, WS_X)) window_attention_kernel(AttnParams p) {
+__global__ void __launch_bounds__(attn_threads(WS_Y, WS_X)) __attribute__((amdgpu_waves_per_eu(2)))
+window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workgroups share a CU
   using Cfg = AttnCfg<WS_Y, WS_X, HD, HAS_BIAS>;
-  constexpr int L = Cfg::L, NW = Cfg::NW, LPAD = Cfg::LPAD, NT = Cfg::NT;
-  constexpr int KROW = Cfg::KROW, VROW = Cfg::VROW, TBL = Cfg::TBL;
+  constexpr int L = Cfg::L, NQ = Cfg::NQ, LPAD = Cfg::LPAD, NT = Cfg::NT, NWAVES = Cfg::NWAVES;
+  constexpr int VROW = Cfg::VROW, TBL = Cfg::TBL;
   constexpr int CH = HD / 8;   // 16-byte chunks per head row
   constexpr int KS = HD / 16;  // k16 steps of QK^T
   constexpr int DB = HD / 32;  // 32-row blocks of O^T
@@ -90,173 +103,241 @@ __global__ void __launch_bounds__(attn_threads(WS_Y, WS_X)) window_attention_ker
     return img_base + (int64_t)Y * W + X;
   };
 
-  // ---- K -> LDS
-  const uint16_t* kbase = p.qkv + inner + head * HD;
-  for (int idx = tid; idx < LPAD * CH; idx += NT) {
-    const int key = idx / CH, c = idx % CH;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (key < L) v = *reinterpret_cast<const u32x4*>(kbase + token_row(key) * ld_qkv + c * 8);
-    *reinterpret_cast<u32x4*>(sK + key * KROW + c * 16) = v;
+  // ---- Q fragments of both query groups of this wave (B operand): lane = query, 8 consecutive d per k16 step.
+  // Issued first: they are needed only after the K / V traffic below.
+  bf16x8 qf[2][KS];
+  int64_t q_tok[2];
+#pragma unroll
+  for (int ps = 0; ps < 2; ++ps) {
+    int qpos = (wave + ps * NWAVES) * 32 + l31;
+    if (qpos >= L) qpos = L - 1;
+    q_tok[ps] = token_row(qpos);
+    const uint16_t* qp = p.qkv + q_tok[ps] * ld_qkv + head * HD + hi * 8;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[ps][s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
   }
-  // ---- V -> registers -> transpose 4 keys x 8 d -> LDS V^T
+
+  // ---- all global loads of the workgroup are issued before the first LDS write (one round trip, not one per
+  // loop iteration): K chunks, V as 4 keys x 8 d per thread, the head's bias column
+  constexpr int K_ITEMS = LPAD * CH, V_ITEMS = (LPAD / 4) * CH;
+  constexpr int KIT = (K_ITEMS + NT - 1) / NT, VIT = (V_ITEMS + NT - 1) / NT, BIT = HAS_BIAS ? (TBL + NT - 1) / NT : 1;
+  const uint16_t* kbase = p.qkv + inner + head * HD;
   const uint16_t* vbase = p.qkv + 2 * inner + head * HD;
-  for (int idx = tid; idx < (LPAD / 4) * CH; idx += NT) {
-    const int kg = idx / CH, c = idx % CH;
-    u32x4 r[4];
+  u32x4 kreg[KIT], vreg[VIT][4];
+  float breg[BIT];
+#pragma unroll
+  for (int it = 0; it < KIT; ++it) {
+    const int idx = tid + it * NT, key = idx / CH, c = idx % CH;
+    kreg[it] = u32x4{0u, 0u, 0u, 0u};
+    if ((K_ITEMS % NT == 0 || idx < K_ITEMS) && (LPAD == L || key < L))  // both compile-time true for full windows
+      kreg[it] = *reinterpret_cast<const u32x4*>(kbase + token_row(key) * ld_qkv + c * 8);
+  }
+#pragma unroll
+  for (int it = 0; it < VIT; ++it) {
+    const int idx = tid + it * NT, kg = idx / CH, c = idx % CH;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      r[j] = u32x4{0u, 0u, 0u, 0u};
-      if (kg * 4 < L) r[j] = *reinterpret_cast<const u32x4*>(vbase + token_row(kg * 4 + j) * ld_qkv + c * 8);
-    }
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {  // word w holds d = 8c + 2w (low half) and 8c + 2w + 1 (high half)
-      u32x2 lo, hi2;
-      lo.x = (r[0][w] & 0xffffu) | (r[1][w] << 16);
-      lo.y = (r[2][w] & 0xffffu) | (r[3][w] << 16);
-      hi2.x = (r[0][w] >> 16) | (r[1][w] & 0xffff0000u);
-      hi2.y = (r[2][w] >> 16) | (r[3][w] & 0xffff0000u);
-      *reinterpret_cast<u32x2*>(sV + (c * 8 + 2 * w) * VROW + kg * 8) = lo;
-      *reinterpret_cast<u32x2*>(sV + (c * 8 + 2 * w + 1) * VROW + kg * 8) = hi2;
+      vreg[it][j] = u32x4{0u, 0u, 0u, 0u};
+      if ((V_ITEMS % NT == 0 || idx < V_ITEMS) && (LPAD == L || kg * 4 < L))
+        vreg[it][j] = *reinterpret_cast<const u32x4*>(vbase + token_row(kg * 4 + j) * ld_qkv + c * 8);
     }
   }
-  // ---- bias column -> LDS 4-vectors
+  if (HAS_BIAS) {
+#pragma unroll
+    for (int it = 0; it < BIT; ++it) {
+      const int j = tid + it * NT;
+      breg[it] = j < TBL ? bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E : 0.f;  // R[j]
+    }
+  }
+  // every load above is in flight before the first LDS write below waits for one of them
+  __builtin_amdgcn_sched_barrier(0);
+  // ---- K -> LDS
+#pragma unroll
+  for (int it = 0; it < KIT; ++it) {
+    const int idx = tid + it * NT, key = idx / CH, c = idx % CH;
+    if (K_ITEMS % NT == 0 || idx < K_ITEMS) *reinterpret_cast<u32x4*>(sK + k_off<HD>(key, c)) = kreg[it];
+  }
+  // ---- V: 4 keys x 8 d register transpose -> LDS as V^T[d][key].  Inside every block of 16 keys the four
+  // key groups are stored in the order 0, 2, 1, 3: the 8 keys one lane needs for a k16 step of PV (4hi..4hi+3
+  // and 8+4hi..8+4hi+3, the accumulator layout of S^T) are then one aligned 16-byte chunk.  Rows are 2*LPAD
+  // bytes, 16-byte chunks XOR-swizzled by the row so that 16 lanes (16 rows, same chunk) hit distinct banks.
+#pragma unroll
+  for (int it = 0; it < VIT; ++it) {
+    const int idx = tid + it * NT, kg = idx / CH, c = idx % CH;
+    if (V_ITEMS % NT == 0 || idx < V_ITEMS) {
+      const int pos = (kg & ~3) | (((kg & 1) << 1) | ((kg >> 1) & 1));  // swap the two middle groups of a 16-key block
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {  // word w holds d = 8c + 2w (low half) and 8c + 2w + 1 (high half)
+        u32x2 lo, hi2;
+        lo.x = (vreg[it][0][w] & 0xffffu) | (vreg[it][1][w] << 16);
+        lo.y = (vreg[it][2][w] & 0xffffu) | (vreg[it][3][w] << 16);
+        hi2.x = (vreg[it][0][w] >> 16) | (vreg[it][1][w] & 0xffff0000u);
+        hi2.y = (vreg[it][2][w] >> 16) | (vreg[it][3][w] & 0xffff0000u);
+        const int d0 = c * 8 + 2 * w, d1 = d0 + 1;
+        *reinterpret_cast<u32x2*>(sV + d0 * VROW + (((pos >> 1) ^ (Cfg::V_SWZ ? (d0 & 15) : 0)) << 4) + (pos & 1) * 8) = lo;
+        *reinterpret_cast<u32x2*>(sV + d1 * VROW + (((pos >> 1) ^ (Cfg::V_SWZ ? (d1 & 15) : 0)) << 4) + (pos & 1) * 8) = hi2;
+      }
+    }
+  }
+  // ---- bias column -> LDS 4-vectors R4[s] = R[s..s+3]
   if (HAS_BIAS) {
     float* sBf = reinterpret_cast<float*>(sB);
-    for (int j = tid; j < TBL; j += NT) {
-      const float r = bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E;  // R[j]
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (j - e >= 0) sBf[(j - e) * 4 + e] = r;  // R4[j-e][e] = R[j]
+    for (int it = 0; it < BIT; ++it) {
+      const int j = tid + it * NT;
+      if (j < TBL) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (j - e >= 0) sBf[(j - e) * 4 + e] = breg[it];  // R4[j-e][e] = R[j]
+      }
     }
     // tail components R4[s][e] with s+e >= TBL are never read by a valid key group
   }
-
-  // ---- Q fragments (B operand): lane = query, 8 consecutive d per k16 step
-  int qpos = wave * 32 + l31;
-  const bool q_valid = qpos < L;
-  if (!q_valid) qpos = L - 1;
-  const int64_t q_tok = token_row(qpos);
-  bf16x8 qf[KS];
-  {
-    const uint16_t* qp = p.qkv + q_tok * ld_qkv + head * HD + hi * 8;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
-  }
   __syncthreads();
 
-  // ---- S^T = K Q^T
-  f32x16 acc[NW];
-#pragma unroll
-  for (int kb = 0; kb < NW; ++kb) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[kb][e] = 0.f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + (kb * 32 + l31) * KROW + (s * 16 + hi * 8) * 2);
-      acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], acc[kb], 0, 0, 0);
-    }
-  }
-  // acc[kb][4g+i] = <k[key], q[query]>, key = 32kb + 8g + 4hi + i, query = qpos
-
-  // ---- cyclic-shift mask: only windows touching the wrapped border carry more than one region
-  const int qiy = qpos / WS_X, qix = qpos % WS_X;
   const bool my = p.use_mask && p.sy > 0 && wy == p.nWy - 1;
   const bool mx = p.use_mask && p.sx > 0 && wx == p.nWx - 1;
-  if (my || mx) {
-    const float neg = -100.0f / p.scale;  // becomes -100 after the scale multiply below
-    const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
-    const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
-#pragma unroll
-    for (int kb = 0; kb < NW; ++kb)
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = kb * 32 + g * 8 + hi * 4 + i;
-          const int kiy = key / WS_X, kix = key % WS_X;
-          const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
-          const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
-          if (ry_k != ry_q || rx_k != rx_q) acc[kb][g * 4 + i] += neg;
-        }
-  }
-
-  // ---- logits in the exp2 domain, row max
   const float c = p.scale * LOG2E;
-  const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
-  float mrow = -INFINITY;
-#pragma unroll
-  for (int kb = 0; kb < NW; ++kb)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int key0 = kb * 32 + g * 8 + hi * 4;
-      const bool valid = (LPAD == L) || key0 < L;
-      f32x4 bv = {0.f, 0.f, 0.f, 0.f};
-      if (HAS_BIAS) {
-        const int kk = valid ? key0 : 0;
-        const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
-        bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float t = fmaf(acc[kb][g * 4 + i], c, bv[i]);
-        if (!valid) t = -INFINITY;
-        acc[kb][g * 4 + i] = t;
-        mrow = fmaxf(mrow, t);
-      }
-    }
-  mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
 
-  // ---- P = exp2(t - max), row sum, pack to bf16 (B operand of PV)
-  float sum = 0.f;
-  uint32_t pk[NW][8];
 #pragma unroll
-  for (int kb = 0; kb < NW; ++kb)
-#pragma unroll
-    for (int h2 = 0; h2 < 8; ++h2) {
-      const float e0 = __builtin_amdgcn_exp2f(acc[kb][2 * h2] - mrow);
-      const float e1 = __builtin_amdgcn_exp2f(acc[kb][2 * h2 + 1] - mrow);
-      sum += e0 + e1;
-      pk[kb][h2] = pack_bf16x2(e0, e1);
-    }
-  sum += __shfl_xor(sum, 32, 64);
-  const float inv = 1.0f / sum;
+  for (int ps = 0; ps < 2; ++ps) {
+    const int qg = wave + ps * NWAVES;
+    if (qg >= NQ) break;  // wave-uniform
+    int qpos = qg * 32 + l31;
+    const bool q_valid = qpos < L;
+    if (!q_valid) qpos = L - 1;
 
-  // ---- O^T = V^T P^T
-  f32x16 o[DB];
+    // ---- S^T = K Q^T
+    f32x16 acc[NQ];
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+    for (int kb = 0; kb < NQ; ++kb) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+      for (int e = 0; e < 16; ++e) acc[kb][e] = 0.f;
 #pragma unroll
-  for (int kb = 0; kb < NW; ++kb)
-#pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2) {
-      // k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3)
-      u32x4 pw = {pk[kb][4 * t2], pk[kb][4 * t2 + 1], pk[kb][4 * t2 + 2], pk[kb][4 * t2 + 3]};
-      const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-      const int kofs = (kb * 32 + t2 * 16 + hi * 4) * 2;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const unsigned char* vp = sV + (db * 32 + l31) * VROW + kofs;
-        const u32x2 v0 = *reinterpret_cast<const u32x2*>(vp);
-        const u32x2 v1 = *reinterpret_cast<const u32x2*>(vp + 16);
-        u32x4 vw = {v0.x, v0.y, v1.x, v1.y};
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vw), pf, o[db], 0, 0, 0);
+      for (int s = 0; s < KS; ++s) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(kb * 32 + l31, s * 2 + hi));
+        acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ps][s], acc[kb], 0, 0, 0);
       }
     }
+    // acc[kb][4g+i] = <k[key], q[query]>, key = 32kb + 8g + 4hi + i, query = qpos
 
-  // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i]
-  if (q_valid) {
-    uint16_t* op = p.out + q_tok * inner + head * HD + hi * 4;
+    // ---- cyclic-shift mask: only windows touching the wrapped border carry more than one region
+    const int qiy = qpos / WS_X, qix = qpos % WS_X;
+    if (my || mx) {
+      const float neg = -100.0f / p.scale;  // becomes -100 after the scale multiply below
+      const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
+      const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = kb * 32 + g * 8 + hi * 4 + i;
+            const int kiy = key / WS_X, kix = key % WS_X;
+            const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
+            const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
+            if (ry_k != ry_q || rx_k != rx_q) acc[kb][g * 4 + i] += neg;
+          }
+    }
+
+    // ---- row max of the logits (exp2 domain).  With a bias the logits are formed here (one FMA each);
+    // without one the max of the raw scores is enough (scale > 0) and the FMA moves into the exp2 argument.
+    float mrow = -INFINITY;
+    if (HAS_BIAS) {
+      const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int key0 = kb * 32 + g * 8 + hi * 4;
+          const bool valid = (LPAD == L) || key0 < L;
+          const int kk = valid ? key0 : 0;
+          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
+          const f32x4 bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+          float t[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            t[i] = fmaf(acc[kb][g * 4 + i], c, bv[i]);
+            if (!valid) t[i] = -INFINITY;
+            acc[kb][g * 4 + i] = t[i];
+          }
+          mrow = fmaxf(fmaxf(mrow, t[0]), t[1]);
+          mrow = fmaxf(fmaxf(mrow, t[2]), t[3]);
+        }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const bool valid = (LPAD == L) || (kb * 32 + g * 8 + hi * 4) < L;
+          if (!valid) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[kb][g * 4 + i] = -INFINITY;
+          }
+          mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4]), acc[kb][g * 4 + 1]);
+          mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4 + 2]), acc[kb][g * 4 + 3]);
+        }
+      mrow *= c;
+    }
+    mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
+
+    // ---- P = exp2(t - max), row sum, pack to bf16 (B operand of PV)
+    float sum = 0.f;
+    uint32_t pk[NQ][8];
+#pragma unroll
+    for (int kb = 0; kb < NQ; ++kb)
+#pragma unroll
+      for (int h2 = 0; h2 < 8; ++h2) {
+        float e0, e1;
+        if (HAS_BIAS) {
+          e0 = __builtin_amdgcn_exp2f(acc[kb][2 * h2] - mrow);
+          e1 = __builtin_amdgcn_exp2f(acc[kb][2 * h2 + 1] - mrow);
+        } else {
+          e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -mrow));
+          e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -mrow));
+        }
+        sum += e0 + e1;
+        pk[kb][h2] = pack_bf16x2(e0, e1);
+      }
+    sum += __shfl_xor(sum, 32, 64);
+    const float inv = __builtin_amdgcn_rcpf(sum);
+
+    // ---- O^T = V^T P^T
+    f32x16 o[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w2;
-        w2.x = pack_bf16x2(o[db][g * 4] * inv, o[db][g * 4 + 1] * inv);
-        w2.y = pack_bf16x2(o[db][g * 4 + 2] * inv, o[db][g * 4 + 3] * inv);
-        *reinterpret_cast<u32x2*>(op + db * 32 + g * 8) = w2;
+      for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < NQ; ++kb)
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        // k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one V^T chunk
+        u32x4 pw = {pk[kb][4 * t2], pk[kb][4 * t2 + 1], pk[kb][4 * t2 + 2], pk[kb][4 * t2 + 3]};
+        const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+        const int chunk = (kb * 32 + t2 * 16) / 8 + hi;  // 16-byte chunk of the row: 8 keys of this lane half
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const int d = db * 32 + l31;
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(sV + d * VROW + ((chunk ^ (Cfg::V_SWZ ? (d & 15) : 0)) << 4));
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, o[db], 0, 0, 0);
+        }
       }
+
+    // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i]
+    if (q_valid) {
+      uint16_t* op = p.out + q_tok[ps] * inner + head * HD + hi * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          u32x2 w2;
+          w2.x = pack_bf16x2(o[db][g * 4] * inv, o[db][g * 4 + 1] * inv);
+          w2.y = pack_bf16x2(o[db][g * 4 + 2] * inv, o[db][g * 4 + 3] * inv);
+          *reinterpret_cast<u32x2*>(op + db * 32 + g * 8) = w2;
+        }
+    }
   }
 }
 

@@ -95,6 +95,9 @@ def main():
     ap.add_argument("--residual", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=32)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one plain 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the whole grid on ONE GPU; --gpus N > 1 is not supported "
@@ -117,6 +120,12 @@ def main():
     x = torch.randn(1, S, wl["cin"], generator=g, device=dev)
     t = (torch.rand(1, generator=g, device=dev) * (math.pi / 2))
 
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     with torch.no_grad():
         for _ in range(args.warmup):
             out = model(x, t)

@@ -24,6 +24,11 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# Bytes that crossed the L2 <-> fabric boundary per launch at the config3 workload (average over the launches of
+# one step), from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a 1 GiB copy kernel; the summary
+# with the commands is profiles/denoiser_step_config3_pmc_traffic.txt.  Not measurable from inside this script.
+PMC_TRAFFIC_BYTES = {"config3": {"gemm_256x256_none_bf16": 26.942e9 + 5.280e9, "gemm_256x256_gelu_bf16": 32.801e9 + 12.743e9,
+                                 "window_attention": 9.556e9 + 3.185e9, "norm_modulate": 3.186e9 + 3.185e9}}
 
 WORKLOADS = {
     # name: grid, dim, heads, head_dim, window, mlp, blocks, in/out channels
@@ -175,7 +180,8 @@ def main():
         dom, a = kernels[dom_tag], agg[dom_tag]
         roofline = {"kernel": NAMES.get(dom_tag, dom_tag),
                     "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                    "frac": dom["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
+                    "frac": dom["tflops"] / PEAK_BF16_TFLOPS,
+                    "traffic": PMC_TRAFFIC_BYTES.get(args.workload, {}).get(dom_tag),
                     "flop_per_launch": a["work"] / a["launches"], "avg_launch_ms": dom["avg_ms"]}
 
     result = {

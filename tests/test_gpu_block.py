@@ -146,3 +146,48 @@ def test_sampler_parity_and_graph_replay(pkg, cuda):
     states = smp.rollout(cond[..., :8].contiguous().to(cuda), 2, torch.Generator(device="cuda").manual_seed(3),
                          extra_cond=cond[..., 8:].contiguous().to(cuda))
     assert len(states) == 2 and all(torch.isfinite(s).all() for s in states)
+
+
+@pytest.mark.parametrize("name,geo", [("config2", dict(dim=1024, heads=16, head_dim=64, mlp_dim=4096)),
+                                      ("config3", dict(dim=1536, heads=24, head_dim=64, mlp_dim=6144))])
+def test_full_grid_block_against_oracle_strips(pkg, cuda, name, geo):
+    """Full 720x1440 grid (1 036 800 tokens, 4 050 windows of 16x16).  A Swin block only mixes tokens inside one
+    window, so a band of window rows of the full-grid result must equal the oracle run on that band alone: rows
+    [16k, 16k+16) for the un-shifted block; rows [16k+8, 16k+24) with a longitude-only shift for the shifted block
+    (no latitude wrap inside the band); the last band of the shifted block wraps in latitude (rows 712..719 + 0..7)
+    and carries the full shift mask."""
+    H, W, ws = 720, 1440, 16
+    cfg = OracleConfig.spec(window_size=(ws, ws), image_shape=(H, W), mod_ways=2, **geo)
+    sd = oracle.init_block_weights(cfg, 17, nontrivial=True)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(1, H * W, cfg.dim, generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    t = torch.randn(1, cfg.dim, generator=torch.Generator().manual_seed(6))
+    for shifted in (False, True):
+        layer = make_layer(pkg, cfg, sd, cuda, shifted)
+        out = layer(x, t.to(cuda))
+        out2 = layer(x, t.to(cuda))
+        torch.cuda.synchronize()
+        assert torch.equal(out, out2)  # deterministic
+        grid_in = x.view(H, W, cfg.dim)
+        grid_out = out.view(H, W, cfg.dim)
+        bands = [0, 22, 44] if not shifted else [0, 21, 44]
+        for k in bands:
+            if not shifted:
+                rows = torch.arange(16 * k, 16 * k + 16)
+                band_cfg = OracleConfig.spec(window_size=(ws, ws), image_shape=(16, W), mod_ways=2, **geo)
+                shift = (0, 0)
+            elif k < 44:
+                rows = torch.arange(16 * k + 8, 16 * k + 24)
+                band_cfg = OracleConfig.spec(window_size=(ws, ws), image_shape=(16, W), mod_ways=2, **geo)
+                shift = (0, 8)
+            else:  # wrapped band: rows 0..23 followed by rows 712..719 form a 32-row image whose half-window roll puts
+                #    rows 8..23 into its first window row and rows 712..719 + 0..7 into its last, masked, window row:
+                #    exactly the first and the last window row of the rolled full grid
+                rows = torch.cat([torch.arange(0, 24), torch.arange(712, 720)])
+                band_cfg = OracleConfig.spec(window_size=(ws, ws), image_shape=(32, W), mod_ways=2, **geo)
+                shift = (8, 8)
+            xin = grid_in[rows.to(cuda)].float().cpu().reshape(1, -1, cfg.dim)
+            ref = oracle.block_forward(band_cfg, sd, xin, t, shift).reshape(len(rows), W, cfg.dim)
+            got = grid_out[rows.to(cuda)].float().cpu()
+            err = rel_l2(got, ref)
+            assert err <= 1e-2, (name, shifted, k, err)

@@ -23,31 +23,35 @@
 namespace aeris {
 
 namespace {
-constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 4;
+constexpr int BM = 256, BN = 256, BK = 32, WM = 2, WN = 4;
 constexpr int NT = WM * WN * 64;          // 512 threads
 constexpr int FM = BM / WM / 32;          // 4
 constexpr int FN = BN / WN / 32;          // 2
-constexpr int A_BYTES = BM * BK * 2;      // 32 KB
-constexpr int B_BYTES = BN * BK * 2;      // 32 KB
-constexpr int STAGE = A_BYTES + B_BYTES;  // 64 KB
-constexpr int RP = NT / 8;                // 64 tile rows per loader pass
-constexpr int A_IT = BM / RP;             // 4
-constexpr int B_IT = BN / RP;             // 4
-constexpr int EPI_OFF = 2 * STAGE;        // wave-private staging, 4 KB per wave
-constexpr int SMEM = 2 * STAGE + 8 * 4096;
+constexpr int A_BYTES = BM * BK * 2;      // 16 KB
+constexpr int B_BYTES = BN * BK * 2;      // 16 KB
+constexpr int STAGE = A_BYTES + B_BYTES;  // 32 KB
+constexpr int NSTAGE = 4;
+constexpr int EPI_OFF = NSTAGE * STAGE;   // wave-private staging, 4 KB per wave
+constexpr int SMEM = NSTAGE * STAGE + 8 * 4096;
 constexpr int GM = 4;                     // row panels per L2 group
+
+// Byte offset of 16-byte chunk `chunk` (0..3) of row `row` in a [rows][32] bf16 k-tile.  A 256-byte line holds four
+// rows; the slot of a chunk inside its line is XORed with the row-pair index, which makes both the ds_read_b128
+// of an MFMA fragment (32 rows x 2 chunks per wave) and the 1 KB row-block writes of the loader conflict-free.
+__device__ __forceinline__ uint32_t tile_off(int row, int chunk) {
+  return (uint32_t)((row >> 2) * 256 + (((((row & 1) << 3) | (((row >> 1) & 1) << 2) | chunk) ^ ((row >> 1) & 7)) << 4));
+}
 }  // namespace
 
 template <int ACT, bool OUT_F32>
 __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams p) {
   constexpr bool SWIGLU = ACT == AERIS_ACT_SWIGLU;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
   const int l31 = lane & 31, hi = lane >> 5;
-  const int lc = tid & 7, lr = tid >> 3;
   const int K = p.K, N = p.N;
   const int KT = K / BK;
 
@@ -69,76 +73,68 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     tile_m = grp * GM + (within - tile_n * gm);
   };
 
-  // ---- loader state (runs two k-tiles ahead of the compute state)
-  const uint16_t* ld_a = nullptr;
-  const uint16_t* ld_b = nullptr;
-  uint32_t a_goff[A_IT], b_goff[B_IT];
-  int ld_r = 0, ld_kt = 0;
+  // ---- loader: global memory -> LDS without passing through registers (buffer_load ... lds, 16 bytes per lane).
+  // One instruction of a wave fills 1 KB of LDS, lane l at byte 16 l: four lines = 16 rows of a k-tile in the
+  // layout of tile_off(), so the lane fetches the chunk which that layout keeps at its LDS slot (four consecutive
+  // lanes fetch the 64 contiguous bytes of one row).  Rows past the end of A or W are outside the buffer
+  // descriptor and arrive as zeros; they only feed rows / columns of C that are never stored.
+  // Per k-tile a wave brings in 32 rows of A (instructions 0, 1) and 32 rows of W (instructions 2, 3).
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int grp = wave_u / WN;
+  uint32_t ld_voff;  // lane part of the source offset (the same for every 16-row block)
+  {
+    const int lb = lane >> 4, pos = lane & 15;
+    const int v = (pos & 7) ^ ((2 * lb) & 7);
+    const int b = v >> 2, cq = (v ^ b) & 3;
+    ld_voff = (uint32_t)((4 * lb + 2 * b + (pos >> 3)) * K * 2 + cq * 16);
+  }
+  const __amdgpu_buffer_rsrc_t rs_w =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.W, 0, (int)((SWIGLU ? 2 : 1) * (int64_t)N * K * 2), 0x00020000);
+  __amdgpu_buffer_rsrc_t rs_a = rs_w;
+  uint32_t ld_brow = 0;  // W row of the first of this wave's 32 rows of the tile
+  int ld_r = 0, ld_kt = 0, ld_stage = 0;
   auto ld_set_tile = [&]() {
     if (ld_r >= n_my) return;
     int tile_m, tile_n;
     decode(ld_r, tile_m, tile_n);
     const int64_t m0 = (int64_t)tile_m * BM;
     const int n0 = tile_n * BN_OUT;
-    const int64_t last = p.M - 1 - m0;
-#pragma unroll
-    for (int i = 0; i < A_IT; ++i) {
-      int64_t r = lr + i * RP;
-      if (r > last) r = last;
-      a_goff[i] = (uint32_t)(r * K + lc * 8);
-    }
-    ld_a = p.A + m0 * K;
-    int first_row = SWIGLU ? 0 : n0;
-#pragma unroll
-    for (int i = 0; i < B_IT; ++i) {
-      const int j = lr + i * RP;
-      int r;
-      if (SWIGLU) {
-        constexpr int WNW = BN / WN;  // columns of the tile owned by one wave: [gate 32 | up 32]
-        const int wv = j / WNW, within = j % WNW;
-        const int oc = n0 + wv * 32 + (within & 31);
-        r = ((within >> 5) ? N : 0) + (oc < N ? oc : N - 1);
-      } else {
-        r = n0 + j;
-        if (r > N - 1) r = N - 1;
-        r -= first_row;
-      }
-      b_goff[i] = (uint32_t)((int64_t)r * K + lc * 8);
-    }
-    ld_b = p.W + (int64_t)first_row * K;
+    int64_t rows = p.M - m0;
+    if (rows > BM) rows = BM;
+    rs_a = __builtin_amdgcn_make_buffer_rsrc((void*)(p.A + m0 * K), 0, (int)(rows * K * 2), 0x00020000);
+    // SwiGLU: tile rows [64 c, 64 c + 64) are the gate rows, then the up rows, of 32 output columns
+    if (SWIGLU) ld_brow = (uint32_t)((wave_u & 1) * N + n0 + (wave_u >> 1) * 32);
+    else ld_brow = (uint32_t)(n0 + wave_u * 32);
   };
-
-  u32x4 ra[A_IT], rb[B_IT];
-  auto issue = [&]() {
+  // part 0: the two A instructions of the loader's current k-tile; part 1: the two W instructions, then advance
+  auto issue = [&](int part) {
     if (ld_r < n_my) {
-      const uint16_t* ab = ld_a + (int64_t)ld_kt * BK;
-      const uint16_t* bb = ld_b + (int64_t)ld_kt * BK;
-#pragma unroll
-      for (int i = 0; i < A_IT; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ab + a_goff[i]);
-#pragma unroll
-      for (int i = 0; i < B_IT; ++i) rb[i] = *reinterpret_cast<const u32x4*>(bb + b_goff[i]);
-      if (++ld_kt == KT) {
-        ld_kt = 0;
-        ++ld_r;
-        ld_set_tile();
+      typedef __attribute__((address_space(3))) void* lds_ptr;
+      unsigned char* sd = smem + (ld_stage & (NSTAGE - 1)) * STAGE + part * A_BYTES + wave_u * 2048;
+      const uint32_t row0 = part ? ld_brow : (uint32_t)(wave_u * 32);
+      const uint32_t so = row0 * (uint32_t)(K * 2) + (uint32_t)ld_kt * (BK * 2);
+      if (part == 0) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)sd, 16, ld_voff, so, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(sd + 1024), 16, ld_voff, so + 16u * (uint32_t)(K * 2), 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)sd, 16, ld_voff, so, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(sd + 1024), 16, ld_voff, so + 16u * (uint32_t)(K * 2), 0, 0);
+        ++ld_stage;
+        if (++ld_kt == KT) {
+          ld_kt = 0;
+          ++ld_r;
+          ld_set_tile();
+        }
       }
     }
-  };
-  const uint32_t w_off = swz_off(lr, lc);
-  auto lstore = [&](int stage) {
-    unsigned char* s = smem + stage * STAGE;
-#pragma unroll
-    for (int i = 0; i < A_IT; ++i) *reinterpret_cast<u32x4*>(s + w_off + i * RP * 128) = ra[i];
-#pragma unroll
-    for (int i = 0; i < B_IT; ++i) *reinterpret_cast<u32x4*>(s + A_BYTES + w_off + i * RP * 128) = rb[i];
   };
 
   // ---- fragment read offsets (per k16 step)
-  uint32_t a_roff[4], b_roff[4];
+  uint32_t a_roff[2], b_roff[2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    a_roff[ks] = swz_off(wm * (BM / WM) + l31, ks * 2 + hi);
-    b_roff[ks] = A_BYTES + swz_off(wn * (BN / WN) + l31, ks * 2 + hi);
+  for (int ks = 0; ks < 2; ++ks) {
+    a_roff[ks] = tile_off(wm * (BM / WM) + l31, ks * 2 + hi);
+    b_roff[ks] = A_BYTES + tile_off(wn * (BN / WN) + l31, ks * 2 + hi);
   }
 
   f32x16 acc[FM][FN];
@@ -297,44 +293,79 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     }
   };
 
-  // ---- flat pipeline over (tile, k-tile): a k-tile is loaded a full step before it is moved to LDS
+  // ---- flat pipeline over (tile, k-tile) with four LDS stages, ping-pong between the two wave groups.
+  // Group 0 (wm = 0, one wave per SIMD) and group 1 (wm = 1, the other wave of each SIMD) run, per k-tile, a
+  // memory slot M (12 ds_read_b128: the fragments of the k-tile) and a compute slot C (16 MFMAs), one slot
+  // apart, every slot ending in a workgroup barrier: while one wave of a SIMD computes, the other one does its
+  // memory work, so the matrix pipe and the LDS are busy at the same time instead of in turns.
+  // Slots are numbered globally: group 0 runs M(q), C(q) in slots 2q, 2q+1, group 1 in 2q+1, 2q+2.  Stage q & 3
+  // is read in slots 2q and 2q+1 and then refilled with k-tile q+4.  Every wave issues its four loads of k-tile
+  // q+3 in its slot M(q) (slots 2q, 2q+1: after the last read of that stage in slot 2q-1), behind its LDS reads:
+  // a load instruction occupies the issuing wave while the CU's address unit takes its 64 addresses, which
+  // would stall the MFMA stream of a compute slot but costs nothing next to the LDS latency of a memory slot.
+  // k-tile q+1 is first read in slot 2q+2: every wave waits for its loads of k-tile q+1 before the barrier
+  // that ends slot 2q+1, with the 8 loads of k-tiles q+2, q+3 allowed to be in flight.  For group 0 that is the
+  // end of C(q), for group 1 the end of M(q).  (Between two tiles both groups insert one idle slot, see below;
+  // it only adds slack.)  Vector memory operations complete in order, so anything the epilogue has issued in between only
+  // makes these waits more conservative; at the end of the list, where fewer loads follow, the wait is for all.
+  // A slot ends in a bare s_barrier: the fences of __syncthreads() would make every wave wait for all of its
+  // outstanding loads into LDS.  What a barrier has to order is stated explicitly with s_waitcnt.
+  constexpr int WAIT_LGKM0 = 0xC07F, WAIT_VM0 = 0x0F70, WAIT_VM8 = 0x0F78, WAIT_VM8_LGKM0 = 0x0078, WAIT_ALL = 0x0070;
   const int total = n_my * KT;
-  int c_r = 0, c_kt = 0;  // compute state
   ld_set_tile();
-  issue();
-  lstore(0);
-  issue();  // k-tile 1 stays in registers until the middle of step 0
+#pragma unroll
+  for (int q = 0; q < 3; ++q) {
+    issue(0);
+    issue(1);
+  }
+  __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   __syncthreads();
-
-  for (int j = 0; j < total; ++j) {
-    const unsigned char* s = smem + (j & 1) * STAGE;
+  int q = 0;  // position in the flat list of k-tiles
+  for (int r = 0; r < n_my; ++r) {
+    // Group 1 runs one slot behind group 0.  The offset is set up anew for every tile (group 1 waits one slot
+    // here, group 0 one slot before its epilogue), so that both groups run their epilogues at the same time:
+    // with the epilogues one slot apart, each would hold up the other group at a barrier.
+    if (grp == 1) __builtin_amdgcn_s_barrier();
+    for (int kt = 0; kt < KT; ++kt, ++q) {
+      const unsigned char* s = smem + (q & (NSTAGE - 1)) * STAGE;
+      const bool more = q + 3 < total;
+      // ---- memory slot: LDS reads first (queued, non-blocking), then the loads of k-tile q+3
+      bf16x8 af[2][FM], bfr[2][FN];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      // the other LDS stage is idle during this step: half way through, move k-tile j+1 (loaded a full step
-      // ago) from the staging registers into it and immediately reuse the registers for the loads of k-tile
-      // j+2.  The wait for the loads overlaps with the MFMAs of the second wave on this SIMD.
-      if (ks == 2 && j + 1 < total) {
-        lstore((j + 1) & 1);
-        issue();
+      for (int k2 = 0; k2 < 2; ++k2) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i) af[k2][i] = *reinterpret_cast<const bf16x8*>(s + a_roff[k2] + i * 32 * 64);
+#pragma unroll
+        for (int jn = 0; jn < FN; ++jn) bfr[k2][jn] = *reinterpret_cast<const bf16x8*>(s + b_roff[k2] + jn * 32 * 64);
       }
-      bf16x8 af[FM], bfr[FN];
+      __builtin_amdgcn_sched_barrier(0);
+      issue(0);
+      issue(1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (grp == 0) __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
+      else if (more) __builtin_amdgcn_s_waitcnt(WAIT_VM8_LGKM0);
+      else __builtin_amdgcn_s_waitcnt(WAIT_ALL);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- compute slot
 #pragma unroll
-      for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(s + a_roff[ks] + i * 32 * 128);
+      for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
-      for (int jn = 0; jn < FN; ++jn) bfr[jn] = *reinterpret_cast<const bf16x8*>(s + b_roff[ks] + jn * 32 * 128);
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int jn = 0; jn < FN; ++jn)
-          acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[jn], af[i], acc[i][jn], 0, 0, 0);
+          for (int jn = 0; jn < FN; ++jn)
+            acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[k2][jn], af[k2][i], acc[i][jn], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (grp == 0) {
+        if (more) __builtin_amdgcn_s_waitcnt(WAIT_VM8);
+        else __builtin_amdgcn_s_waitcnt(WAIT_VM0);
+      }
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __syncthreads();
-    if (++c_kt == KT) {
-      epilogue(c_r);
-      zero_acc();
-      c_kt = 0;
-      ++c_r;
-    }
+    if (grp == 0) __builtin_amdgcn_s_barrier();
+    epilogue(r);
+    zero_acc();
   }
 }
 

@@ -148,54 +148,115 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   };
   zero_acc();
 
-  // ---- epilogue of the tile whose accumulators are complete
+  // ---- epilogue of the tile whose accumulators are complete.
+  // Vector memory operations of a wave complete in order, so a wait for a load also waits for every store issued
+  // before it.  The epilogue therefore loads everything it can ahead of its stores: the per-column operands
+  // (bias, gate) once per tile, the residual rows of the next 32-row block before the stores of the current one.
   unsigned char* stg = smem + EPI_OFF + wave * 4096;
   const int rrow = lane >> 3, rch = lane & 7;  // read-back mapping: row rrow + 8*it, 16-byte chunk rch
   auto epilogue = [&](int r_done) {
     int tile_m, tile_n;
     decode(r_done, tile_m, tile_n);
-    const int64_t m_base = (int64_t)tile_m * BM + wm * (BM / WM);
-    const int n_wave = tile_n * BN_OUT + wn * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-      const int64_t m_lane = m_base + i * 32 + l31;  // row of the fragment values this lane holds
-      const float* gate_row = nullptr;
-      if (p.gate) {
-        int64_t mm = m_lane < p.M ? m_lane : p.M - 1;
-        gate_row = p.gate + (p.gate_batch_stride ? (mm / p.rows_per_batch) * p.gate_batch_stride : 0);
+    const int64_t m_base = (int64_t)tile_m * BM + grp * (BM / WM);
+    const int n_wave = tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
+    constexpr int NJ = SWIGLU ? 1 : FN;
+
+    // gate: one row of p.gate per batch.  A tile whose rows are all in one batch (the usual case) loads its gate
+    // columns once; otherwise every lane looks up the row of its own fragment row.
+    const float* gate_tile = nullptr;
+    bool gate_per_lane = false;
+    if (p.gate) {
+      if (p.gate_batch_stride == 0) {
+        gate_tile = p.gate;
+      } else {
+        int64_t last = m_base + BM / WM - 1;
+        if (last > p.M - 1) last = p.M - 1;
+        const int64_t b0 = m_base / p.rows_per_batch, b1 = last / p.rows_per_batch;
+        if (b0 == b1) gate_tile = p.gate + b0 * p.gate_batch_stride;
+        else gate_per_lane = true;
       }
-      // stage 1: bias / activation / gate on one 32 x 32 fragment, 4 consecutive n per g (N % 4 == 0, so a
-      // group of 4 is entirely inside or entirely outside the matrix)
-      auto fragment = [&](int j, float (&v)[4][4]) {
+    }
+    // fragment columns of this lane: 4 consecutive n per (j, g); N % 4 == 0, so a group of 4 is entirely inside
+    // or entirely outside the matrix (outside: clamped, computed, never stored)
+    u32x2 bq[NJ][4], bq1[NJ][4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          int n = n_wave + j * 32 + g * 8 + hi * 4;
-          if (n >= N) n = N - 4;  // clamped group: computed but never stored
-          f32x4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f}, gt = {1.f, 1.f, 1.f, 1.f};
-          if (p.bias) {
-            const u32x2 r = *reinterpret_cast<const u32x2*>(p.bias + n);
-            b0 = f32x4{bf16_lo(r.x), bf16_hi(r.x), bf16_lo(r.y), bf16_hi(r.y)};
-            if (SWIGLU) {
-              const u32x2 r1 = *reinterpret_cast<const u32x2*>(p.bias + N + n);
-              b1 = f32x4{bf16_lo(r1.x), bf16_hi(r1.x), bf16_lo(r1.y), bf16_hi(r1.y)};
-            }
-          }
-          if (gate_row) gt = *reinterpret_cast<const f32x4*>(gate_row + n);
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float x = acc[i][j][g * 4 + e] + b0[e];
-            if (SWIGLU) x = silu_f(x) * (acc[i][1][g * 4 + e] + b1[e]);
-            else if (ACT == AERIS_ACT_GELU) x = OUT_F32 ? gelu_erf_f(x) : gelu_bf16_f(x);
-            v[g][e] = x * gt[e];
+      for (int g = 0; g < 4; ++g) {
+        int n = n_wave + j * 32 + g * 8 + hi * 4;
+        if (n >= N) n = N - 4;
+        bq[j][g] = u32x2{0u, 0u};
+        bq1[j][g] = u32x2{0u, 0u};
+        if (p.bias) {
+          bq[j][g] = *reinterpret_cast<const u32x2*>(p.bias + n);
+          if (SWIGLU) bq1[j][g] = *reinterpret_cast<const u32x2*>(p.bias + N + n);
+        }
+      }
+
+    // stage 1: bias / activation on the 32 x 32 fragments of row block i, column block j.  The gate is applied
+    // after the staging, where a lane holds consecutive columns of one row and needs far fewer gate registers.
+    auto fragment = [&](int i, int j, float (&v)[4][4]) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b0 = {bf16_lo(bq[j][g].x), bf16_hi(bq[j][g].x), bf16_lo(bq[j][g].y), bf16_hi(bq[j][g].y)};
+        const f32x4 b1 = {bf16_lo(bq1[j][g].x), bf16_hi(bq1[j][g].x), bf16_lo(bq1[j][g].y), bf16_hi(bq1[j][g].y)};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float x = acc[i][j][g * 4 + e] + b0[e];
+          if (SWIGLU) x = silu_f(x) * (acc[i][1][g * 4 + e] + b1[e]);
+          else if (ACT == AERIS_ACT_GELU) x = OUT_F32 ? gelu_erf_f(x) : gelu_bf16_f(x);
+          v[g][e] = x;
+        }
+      }
+    };
+    auto gate_row_of = [&](int64_t m) {  // slow path: the tile straddles a batch boundary
+      if (m > p.M - 1) m = p.M - 1;
+      return p.gate + (m / p.rows_per_batch) * p.gate_batch_stride;
+    };
+
+    if (!OUT_F32) {
+      // stage 2 (bf16 C): a whole 32 x 64 (SwiGLU: 32 x 32) block through LDS, rows of 128 B, chunk-swizzled; it
+      // is read back as 16-byte chunks, 8 lanes per row, and C / residual are accessed as full row segments
+      constexpr int CHUNKS = SWIGLU ? 4 : 8;  // 16-byte chunks (8 columns) per staged row
+      const int n = n_wave + rch * 8;
+      const bool col_ok = rch < CHUNKS && n < N;
+      const bool full = n + 8 <= N;  // N % 4 == 0: a chunk is whole or exactly its first half is inside
+      // residual: 16 bytes (bf16) or 2 x 16 bytes (f32) per lane and row, from an address that is always valid:
+      // rows are clamped to M - 1, a half chunk reads the 4 columns before it as well (bf16) or its first half
+      // twice (f32)
+      int n_ld = n;
+      if (!col_ok) n_ld = n_wave;
+      else if (!full && p.res_dtype == AERIS_BF16) n_ld = n - 4;
+      const bool upper = col_ok && !full;  // bf16: the wanted 4 columns are the upper half of what was loaded
+      const int n_g = col_ok ? n : n_wave;
+      f32x4 gt0 = {1.f, 1.f, 1.f, 1.f}, gt1 = {1.f, 1.f, 1.f, 1.f};
+      if (gate_tile) {
+        gt0 = *reinterpret_cast<const f32x4*>(gate_tile + n_g);
+        gt1 = *reinterpret_cast<const f32x4*>(gate_tile + n_g + (full ? 4 : 0));
+      }
+      u32x4 rq[4][2];
+      auto load_res = [&](int i) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          int64_t m = m_base + i * 32 + rrow + 8 * it;
+          if (m > p.M - 1) m = p.M - 1;
+          const int64_t off = m * p.ldc + n_ld;
+          if (p.res_dtype == AERIS_BF16) {
+            rq[it][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
+          } else {
+            const float* rp = reinterpret_cast<const float*>(p.residual) + off;
+            rq[it][0] = *reinterpret_cast<const u32x4*>(rp);
+            rq[it][1] = *reinterpret_cast<const u32x4*>(rp + (full ? 4 : 0));
           }
         }
       };
-      if (!OUT_F32) {
-        // stage 2 (bf16 C): whole 32 x 64 (SwiGLU: 32 x 32) block through LDS, rows of 128 B, chunk-swizzled
+      if (p.res_dtype >= 0) load_res(0);
 #pragma unroll
-        for (int j = 0; j < (SWIGLU ? 1 : FN); ++j) {
+      for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
           float v[4][4];
-          fragment(j, v);
+          fragment(i, j, v);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             u32x2 w2 = {pack_bf16x2(v[g][0], v[g][1]), pack_bf16x2(v[g][2], v[g][3])};
@@ -205,89 +266,124 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        constexpr int CHUNKS = SWIGLU ? 4 : 8;  // 16-byte chunks (8 columns) per staged row
+        u32x4 out[4];
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
           const int row = rrow + 8 * it;
-          const int64_t m = m_base + i * 32 + row;
-          const int n = n_wave + rch * 8;
-          if (rch < CHUNKS && m < p.M && n < N) {
-            const u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
-            const int64_t off = m * p.ldc + n;
-            const bool full = n + 8 <= N;  // N % 4 == 0: a chunk is whole or exactly half inside
-            uint16_t* cp = reinterpret_cast<uint16_t*>(p.C) + off;
-            if (p.res_dtype < 0) {
-              if (full) *reinterpret_cast<u32x4*>(cp) = w4;
-              else *reinterpret_cast<u32x2*>(cp) = u32x2{w4.x, w4.y};
-            } else {
-              float o[8];
+          u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+          if (p.gate || p.res_dtype >= 0) {
+            float o[8];
 #pragma unroll
-              for (int e = 0; e < 4; ++e) { o[2 * e] = bf16_lo(w4[e]); o[2 * e + 1] = bf16_hi(w4[e]); }
-              if (p.res_dtype == AERIS_BF16) {
-                const uint16_t* rp = reinterpret_cast<const uint16_t*>(p.residual) + off;
-                if (full) {
-                  const u32x4 r4 = *reinterpret_cast<const u32x4*>(rp);
+            for (int e = 0; e < 4; ++e) { o[2 * e] = bf16_lo(w4[e]); o[2 * e + 1] = bf16_hi(w4[e]); }
+            if (gate_per_lane) {
+              const float* gr = gate_row_of(m_base + i * 32 + row);
+              gt0 = *reinterpret_cast<const f32x4*>(gr + n_g);
+              gt1 = *reinterpret_cast<const f32x4*>(gr + n_g + (full ? 4 : 0));
+            }
+            if (p.gate) {
 #pragma unroll
-                  for (int e = 0; e < 4; ++e) { o[2 * e] += bf16_lo(r4[e]); o[2 * e + 1] += bf16_hi(r4[e]); }
-                } else {
-                  const u32x2 r2 = *reinterpret_cast<const u32x2*>(rp);
-                  o[0] += bf16_lo(r2.x); o[1] += bf16_hi(r2.x); o[2] += bf16_lo(r2.y); o[3] += bf16_hi(r2.y);
-                }
-              } else {
-                const float* rp = reinterpret_cast<const float*>(p.residual) + off;
-                const f32x4 r0 = *reinterpret_cast<const f32x4*>(rp);
-                o[0] += r0.x; o[1] += r0.y; o[2] += r0.z; o[3] += r0.w;
-                if (full) {
-                  const f32x4 r1 = *reinterpret_cast<const f32x4*>(rp + 4);
-                  o[4] += r1.x; o[5] += r1.y; o[6] += r1.z; o[7] += r1.w;
-                }
-              }
-              if (full) {
-                u32x4 c4 = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
-                *reinterpret_cast<u32x4*>(cp) = c4;
-              } else {
-                u32x2 c2 = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
-                *reinterpret_cast<u32x2*>(cp) = c2;
+              for (int e = 0; e < 4; ++e) { o[e] *= gt0[e]; o[4 + e] *= gt1[e]; }
+            }
+            if (p.res_dtype == AERIS_BF16) {
+              u32x4 r4 = rq[it][0];
+              if (upper) { r4.x = r4.z; r4.y = r4.w; }
+#pragma unroll
+              for (int e = 0; e < 4; ++e) { o[2 * e] += bf16_lo(r4[e]); o[2 * e + 1] += bf16_hi(r4[e]); }
+            } else if (p.res_dtype == AERIS_F32) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                o[e] += __uint_as_float(rq[it][0][e]);
+                o[4 + e] += __uint_as_float(rq[it][1][e]);
               }
             }
+            w4 = u32x4{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
           }
+          out[it] = w4;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-      } else {
-        // stage 2 (f32 C): 32 x 32 block per fragment column j, rows of 128 B (32 floats)
+        if (p.res_dtype >= 0 && i + 1 < FM) load_res(i + 1);  // ahead of the stores below
 #pragma unroll
-        for (int j = 0; j < (SWIGLU ? 1 : FN); ++j) {
-          float v[4][4];
-          fragment(j, v);
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            f32x4 w4 = {v[g][0], v[g][1], v[g][2], v[g][3]};
-            *reinterpret_cast<f32x4*>(stg + l31 * 128 + (((g * 2 + hi) ^ (l31 & 7)) << 4)) = w4;
+        for (int it = 0; it < 4; ++it) {
+          const int64_t m = m_base + i * 32 + rrow + 8 * it;
+          if (col_ok && m < p.M) {
+            uint16_t* cp = reinterpret_cast<uint16_t*>(p.C) + m * p.ldc + n;
+            if (full) *reinterpret_cast<u32x4*>(cp) = out[it];
+            else *reinterpret_cast<u32x2*>(cp) = u32x2{out[it].x, out[it].y};
           }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+      }
+    } else {
+      // stage 2 (f32 C): one 32 x 32 block per fragment, rows of 128 B (32 floats), 4 floats per lane and row
+      constexpr int UNITS = FM * NJ;
+      u32x4 rq[4];
+      auto unit_col = [&](int u) { return n_wave + (u % NJ) * 32 + rch * 4; };
+      f32x4 gt[NJ];
 #pragma unroll
-          for (int it = 0; it < 4; ++it) {
-            const int row = rrow + 8 * it;
-            const int64_t m = m_base + i * 32 + row;
-            const int n = n_wave + j * 32 + rch * 4;
-            if (m < p.M && n < N) {
-              f32x4 o = *reinterpret_cast<const f32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
-              const int64_t off = m * p.ldc + n;
-              if (p.res_dtype == AERIS_BF16) {
-                const u32x2 r2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
-                o.x += bf16_lo(r2.x); o.y += bf16_hi(r2.x); o.z += bf16_lo(r2.y); o.w += bf16_hi(r2.y);
-              } else if (p.res_dtype == AERIS_F32) {
-                const f32x4 r4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.residual) + off);
-                o.x += r4.x; o.y += r4.y; o.z += r4.z; o.w += r4.w;
-              }
-              *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + off) = o;
-            }
+      for (int j = 0; j < NJ; ++j) {
+        int n = unit_col(j);
+        if (n >= N) n = N - 4;
+        gt[j] = f32x4{1.f, 1.f, 1.f, 1.f};
+        if (gate_tile) gt[j] = *reinterpret_cast<const f32x4*>(gate_tile + n);
+      }
+      auto load_res = [&](int u) {
+        const int i = u / NJ;
+        int n = unit_col(u);
+        if (n >= N) n = N - 4;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          int64_t m = m_base + i * 32 + rrow + 8 * it;
+          if (m > p.M - 1) m = p.M - 1;
+          const int64_t off = m * p.ldc + n;
+          if (p.res_dtype == AERIS_BF16) {
+            const u32x2 r2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
+            rq[it] = u32x4{r2.x, r2.y, 0u, 0u};
+          } else {
+            rq[it] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.residual) + off);
           }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
+        }
+      };
+      if (p.res_dtype >= 0) load_res(0);
+#pragma unroll
+      for (int u = 0; u < UNITS; ++u) {
+        const int i = u / NJ, j = u % NJ;
+        float v[4][4];
+        fragment(i, j, v);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x4 w4 = {v[g][0], v[g][1], v[g][2], v[g][3]};
+          *reinterpret_cast<f32x4*>(stg + l31 * 128 + (((g * 2 + hi) ^ (l31 & 7)) << 4)) = w4;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        f32x4 out[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int row = rrow + 8 * it;
+          f32x4 o = *reinterpret_cast<const f32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+          if (gate_per_lane) {
+            int n = unit_col(u);
+            if (n >= N) n = N - 4;
+            gt[j] = *reinterpret_cast<const f32x4*>(gate_row_of(m_base + i * 32 + row) + n);
+          }
+          if (p.gate) o *= gt[j];
+          if (p.res_dtype == AERIS_BF16) {
+            o.x += bf16_lo(rq[it].x); o.y += bf16_hi(rq[it].x); o.z += bf16_lo(rq[it].y); o.w += bf16_hi(rq[it].y);
+          } else if (p.res_dtype == AERIS_F32) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] += __uint_as_float(rq[it][e]);
+          }
+          out[it] = o;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (p.res_dtype >= 0 && u + 1 < UNITS) load_res(u + 1);  // ahead of the stores below
+        const int n = unit_col(u);
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int64_t m = m_base + i * 32 + rrow + 8 * it;
+          if (m < p.M && n < N) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + m * p.ldc + n) = out[it];
         }
       }
     }

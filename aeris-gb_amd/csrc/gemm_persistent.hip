@@ -1,21 +1,18 @@
-// Persistent bf16 MFMA GEMM for gfx950, 256x256x64 tiles:  C[M,N] = epilogue(A[M,K] * W[N,K]^T)
+// Persistent bf16 MFMA GEMM for gfx950, 256x256 output tiles, k-tiles of 32:  C[M,N] = epilogue(A[M,K] * W[N,K]^T)
 //
-// Same fragment layout and LDS swizzle as the plain tile kernel (gemm.hip), restructured around the
-// two things that bound it on MI355X: the latency of the global loads of a k-tile (L2 misses of a
-// k-tile stall the whole workgroup at the barrier) and the un-overlapped prologue / epilogue of
-// every tile when only one workgroup fits a CU.
-//   - one workgroup per CU slot walks a list of tiles (persistent); the loop runs over the flat
-//     sequence (tile, k-tile), so the loads of the next tile's first k-tiles are already in flight
-//     while the epilogue of the current tile runs
-//   - global loads of k-tile j+2 are issued in the middle of step j, right after the staging registers
-//     have been drained into the idle LDS stage (k-tile j+1): a load has a full step to arrive (two LDS
-//     stages, one barrier per k-tile)
-//   - tiles are ordered so that the workgroups resident on one XCD (blockIdx % 8) cover a
-//     contiguous chunk, 4 row panels x all column tiles at a time: few distinct A / W k-slices per
-//     step compete for that XCD's 4 MB L2
-//   - the epilogue goes through a wave-private 4 KB LDS staging area: fragments (4 consecutive n per
-//     lane) are written swizzled, read back row-contiguous, and C / residual are accessed as full
-//     128-byte row segments (8 lanes x 16 B)
+// Same fragment layout as the plain tile kernel (gemm.hip), built around what bounds it on MI355X:
+//   - global loads go straight into LDS (buffer_load ... lds): no staging registers, no ds_write, and the lane ->
+//     address map of the load is the inverse of the LDS swizzle, so the tile lands in the layout the fragment reads want
+//   - four LDS stages of 32 KB; loads run three k-tiles ahead over the flat sequence (tile, k-tile), so the next
+//     tile's first k-tiles are in flight while the epilogue of the current tile runs (one workgroup per CU, persistent)
+//   - the two waves of a SIMD alternate memory slots (LDS fragment reads + load issue) and compute slots (16 MFMAs):
+//     a load instruction holds the issuing wave until the CU's address unit has taken its 64 addresses, which would
+//     stall the MFMA stream if the computing wave issued it
+//   - tiles are ordered so that the workgroups resident on one XCD (blockIdx % 8) cover a contiguous chunk, 4 row
+//     panels x all column tiles at a time: few distinct A / W k-slices per step compete for that XCD's 4 MB L2
+//   - the epilogue goes through a wave-private 4 KB LDS staging area: fragments (4 consecutive n per lane) are
+//     written swizzled, read back row-contiguous, and C / residual are accessed as full row segments (8 lanes x 16 B);
+//     its loads are issued ahead of its stores because vector memory operations complete in order
 #include "common.h"
 #include "gemm_common.h"
 #include "kernels.h"

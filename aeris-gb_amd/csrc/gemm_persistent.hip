@@ -150,28 +150,59 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     b_roff[ks] = swz_off(wn * (BN / WN) + l31, ks * 2 + hi);
   }
 
+  // ---- accumulators.  They start a tile at the bias instead of zero: the bias add costs nothing that way.
+  // A lane's fragment columns are 4 consecutive n per (j, g): n = first column of the wave + 32 j + 8 g + 4 hi.
+  // N % 4 == 0, so a group of 4 is entirely inside or entirely outside the matrix (outside: clamped, computed,
+  // never stored).
+  constexpr int NJ = SWIGLU ? 1 : FN;
   f32x16 acc[FM][FN];
-  auto zero_acc = [&]() {
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto wave_col0 = [&](int r) {  // first output column of this wave in tile r of the list
+    int tile_m, tile_n;
+    decode(r, tile_m, tile_n);
+    return tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);
   };
-  zero_acc();
+  auto load_bias = [&](int r, u32x2 (&bq)[FN][4]) {  // [SwiGLU: j = 0 gate bias, j = 1 up bias]
+    const int n_wave = wave_col0(r);
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int n = n_wave + (SWIGLU ? 0 : j * 32) + g * 8 + hi * 4;
+        if (n >= N) n = N - 4;
+        bq[j][g] = u32x2{0u, 0u};
+        if (p.bias) bq[j][g] = *reinterpret_cast<const u32x2*>(p.bias + (SWIGLU ? j * N : 0) + n);
+      }
+  };
+  auto init_acc = [&](const u32x2 (&bq)[FN][4]) {
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float b[4] = {bf16_lo(bq[j][g].x), bf16_hi(bq[j][g].x), bf16_lo(bq[j][g].y), bf16_hi(bq[j][g].y)};
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] = b[e];
+      }
+  };
+  {
+    u32x2 bq[FN][4];
+    load_bias(0, bq);
+    init_acc(bq);
+  }
 
   // ---- epilogue of the tile whose accumulators are complete.
   // Vector memory operations of a wave complete in order, so a wait for a load also waits for every store issued
   // before it.  The epilogue therefore loads everything it can ahead of its stores: the per-column operands
-  // (bias, gate) once per tile, the residual rows of the next 32-row block before the stores of the current one.
+  // (gate) once per tile, the residual rows of the next 32-row block before the stores of the current one, the
+  // bias of the next tile (for its accumulators) at the very start.
   const int rrow = lane >> 3, rch = lane & 7;  // read-back mapping: row rrow + 8*it, 16-byte chunk rch
   auto epilogue = [&](int r_done) {
     int tile_m, tile_n;
     decode(r_done, tile_m, tile_n);
     const int64_t m_base = (int64_t)tile_m * BM + grp * (BM / WM);
     const int n_wave = tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
-    constexpr int NJ = SWIGLU ? 1 : FN;
+    u32x2 bq_next[FN][4];  // loaded ahead of the last block's stores, used after them
     // Staging area of this wave, 32 rows of 128 B: the A stage that the loader fills next is idle during the
     // epilogue, and the 4 KB of it that this wave's own loads will fill are written by nobody else.
     unsigned char* stg = smem + la_stage * A_BYTES + wave_u * 4096;
@@ -191,34 +222,16 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         else gate_per_lane = true;
       }
     }
-    // fragment columns of this lane: 4 consecutive n per (j, g); N % 4 == 0, so a group of 4 is entirely inside
-    // or entirely outside the matrix (outside: clamped, computed, never stored)
-    u32x2 bq[NJ][4], bq1[NJ][4];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        int n = n_wave + j * 32 + g * 8 + hi * 4;
-        if (n >= N) n = N - 4;
-        bq[j][g] = u32x2{0u, 0u};
-        bq1[j][g] = u32x2{0u, 0u};
-        if (p.bias) {
-          bq[j][g] = *reinterpret_cast<const u32x2*>(p.bias + n);
-          if (SWIGLU) bq1[j][g] = *reinterpret_cast<const u32x2*>(p.bias + N + n);
-        }
-      }
-
-    // stage 1: bias / activation on the 32 x 32 fragments of row block i, column block j.  The gate is applied
-    // after the staging, where a lane holds consecutive columns of one row and needs far fewer gate registers.
+    // stage 1: activation on the 32 x 32 fragments of row block i, column block j (the bias is in the
+    // accumulators already).  The gate is applied after the staging, where a lane holds consecutive columns of
+    // one row and needs far fewer gate registers.
     auto fragment = [&](int i, int j, float (&v)[4][4]) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const f32x4 b0 = {bf16_lo(bq[j][g].x), bf16_hi(bq[j][g].x), bf16_lo(bq[j][g].y), bf16_hi(bq[j][g].y)};
-        const f32x4 b1 = {bf16_lo(bq1[j][g].x), bf16_hi(bq1[j][g].x), bf16_lo(bq1[j][g].y), bf16_hi(bq1[j][g].y)};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float x = acc[i][j][g * 4 + e] + b0[e];
-          if (SWIGLU) x = silu_f(x) * (acc[i][1][g * 4 + e] + b1[e]);
+          float x = acc[i][j][g * 4 + e];
+          if (SWIGLU) x = silu_f(x) * acc[i][1][g * 4 + e];
           else if (ACT == AERIS_ACT_GELU) x = OUT_F32 ? gelu_erf_f(x) : gelu_bf16_f(x);
           v[g][e] = x;
         }
@@ -317,7 +330,11 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (p.res_dtype >= 0 && i + 1 < FM) load_res(i + 1);  // ahead of the stores below
+        if (i + 1 < FM) {
+          if (p.res_dtype >= 0) load_res(i + 1);  // ahead of the stores below
+        } else if (r_done + 1 < n_my) {
+          load_bias(r_done + 1, bq_next);
+        }
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
           const int64_t m = m_base + i * 32 + rrow + 8 * it;
@@ -393,7 +410,11 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (p.res_dtype >= 0 && u + 1 < UNITS) load_res(u + 1);  // ahead of the stores below
+        if (u + 1 < UNITS) {
+          if (p.res_dtype >= 0) load_res(u + 1);  // ahead of the stores below
+        } else if (r_done + 1 < n_my) {
+          load_bias(r_done + 1, bq_next);
+        }
         const int n = unit_col(u);
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -402,6 +423,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         }
       }
     }
+    if (r_done + 1 < n_my) init_acc(bq_next);
   };
 
   // ---- flat pipeline over (tile, k-tile), ping-pong between the two wave groups.
@@ -481,8 +503,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       }
     }
     if (grp == 0) __builtin_amdgcn_s_barrier();
-    epilogue(r);
-    zero_acc();
+    epilogue(r);  // leaves the accumulators at the bias of the next tile
   }
 }
 

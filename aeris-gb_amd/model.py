@@ -192,7 +192,8 @@ class Attention(nn.Module):
     def core(self, y, shift=(0, 0), out=None):
         """y bf16 [b, n, d] -> attention output before ``wo`` (bf16 [b*n, inner])."""
         b, n, _ = y.shape
-        qkv = ops.gemm(y, self.to_qkv.weight, self.to_qkv.bias)
+        qkv = ops.gemm(y, self.to_qkv.weight, self.to_qkv.bias,
+                       out=ops.workspace("qkv", (b, n, self.to_qkv.weight.shape[0]), torch.bfloat16, y.device))
         return ops.window_attention(qkv.view(b * n, -1), b, self.image_shape, self.heads, self.head_dim,
                                     self.window_size, shift, self.relative_position_bias_table,
                                     self.shift_mask and (shift[0] > 0 or shift[1] > 0), self.scale, out=out)
@@ -280,8 +281,9 @@ class SwinLayer(nn.Module):
                 s1, c1, g1, s2, c2, g2 = parts  # model.py:399
             else:
                 s1, c1, s2, c2 = parts
-        y = _norm_call(o, n1, x, s1, c1)
-        a = attn.core(y, shift)
+        # intermediates live in shared scratch buffers (ops.workspace); only `out` is returned
+        y = _norm_call(o, n1, x, s1, c1, out=ops.workspace("norm", (b, n, d), torch.bfloat16, x.device))
+        a = attn.core(y, shift, out=ops.workspace("attn", (b * n, attn.wo.weight.shape[1]), torch.bfloat16, x.device))
         if branches is not None:
             branches["attn"] = ops.gemm(a, attn.wo.weight, attn.wo.bias).view(b, n, d)
         if out is None:
@@ -289,10 +291,12 @@ class SwinLayer(nn.Module):
         ops.gemm(a, attn.wo.weight, attn.wo.bias, gate=g1, residual=x, rows_per_batch=n, out=out)
         z = _norm_call(o, n2, out, s2, c2, out=y)
         if o.mlp == "swiglu":
-            h = ops.gemm(z, ff.w1.weight, act="swiglu")
+            h = ops.gemm(z, ff.w1.weight, act="swiglu",
+                         out=ops.workspace("hidden", (b, n, ff.w1.weight.shape[0] // 2), torch.bfloat16, x.device))
             w_dn, b_dn = ff.w2.weight, None
         else:
-            h = ops.gemm(z, ff.fc1.weight, ff.fc1.bias, act="gelu")
+            h = ops.gemm(z, ff.fc1.weight, ff.fc1.bias, act="gelu",
+                         out=ops.workspace("hidden", (b, n, ff.fc1.weight.shape[0]), torch.bfloat16, x.device))
             w_dn, b_dn = ff.fc2.weight, ff.fc2.bias
         if branches is not None:
             branches["mlp"] = ops.gemm(h, w_dn, b_dn).view(b, n, d)

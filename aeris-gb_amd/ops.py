@@ -57,6 +57,28 @@ def gemm_uses_big_tiles(M, N, act=None):
     return M >= 256 and (N % bn == 0 or N >= 4 * bn) and ((M + 255) // 256) * ((N + bn - 1) // bn) >= 256 and N % 4 == 0
 
 
+_WORKSPACE = {}
+_RETIRED = []  # outgrown buffers stay allocated: a captured HIP graph may still point into them
+
+
+def workspace(tag: str, shape, dtype, device) -> torch.Tensor:
+    """Reusable scratch tensor for an intermediate that never leaves the block (normalised tokens, qkv, attention
+    output, MLP hidden).  One buffer per (tag, device, dtype), grown on demand and never freed, so eager calls and
+    captured graphs share it instead of each holding a pool of their own (at batch 4 on the 720x1440 grid the four
+    intermediates are 115 GB).  Calls that use the same tag must be ordered on one stream."""
+    n = 1
+    for d in shape:
+        n *= int(d)
+    key = (tag, str(device), dtype)
+    buf = _WORKSPACE.get(key)
+    if buf is None or buf.numel() < n:
+        if buf is not None:
+            _RETIRED.append(buf)
+        buf = torch.empty(n, dtype=dtype, device=device)
+        _WORKSPACE[key] = buf
+    return buf[:n].view(*shape)
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 

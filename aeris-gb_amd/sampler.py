@@ -62,6 +62,7 @@ class TrigFlowSampler:
                 self.sample(self._cond, self._lat)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        torch.cuda.empty_cache()  # the warm-up's cached blocks would sit next to the graph's own pool
         self._graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self._graph):
             self._out = self.sample(self._cond, self._lat)

@@ -36,6 +36,10 @@ WORKLOADS = {
                     cin=138, cout=69, desc="configs[3]: full denoiser step, 720x1440 grid, 24 blocks, dim 1536, 24x64 heads, 16x16 windows"),
     "config2": dict(image_shape=(720, 1440), dim=1024, heads=16, head_dim=64, window=16, mlp_dim=4096, blocks=1,
                     cin=138, cout=69, desc="configs[2]-shaped denoiser with ONE shifted block, dim 1024, 16x64 heads"),
+    "config4": dict(image_shape=(720, 1440), dim=1536, heads=24, head_dim=64, window=16, mlp_dim=6144, blocks=24,
+                    cin=138, cout=69, rollout=True,
+                    desc="configs[4]: ensemble rollout with the configs[3] denoiser, members as batch, Heun ODE sampler "
+                         "replayed as one HIP graph per forecast step"),
     "config1": dict(image_shape=(180, 360), dim=512, heads=8, head_dim=64, window=12, mlp_dim=2048, blocks=2,
                     cin=138, cout=69, desc="configs[1]-shaped denoiser, 180x360 grid, 2 blocks, dim 512, 12x12 windows"),
 }
@@ -59,6 +63,57 @@ def build_model(pkg, torch, wl, device, residual_dtype):
             else:
                 p.fill_(1.0)
     return model
+
+
+def run_rollout(args, pkg, torch, wl, model, dev):
+    """configs[4]: `--steps` autoregressive forecast steps (a step = one forecast step = 2n-1 denoiser calls on a
+    batch of `--ensemble` members), the sampler loop replayed as a HIP graph.  No cpu_baseline leg (N/A: minutes of
+    GPU time per step); the roofline object is the dominant GEMM of one eager denoiser call at this batch."""
+    H, W = wl["image_shape"]
+    S, B, C = H * W, args.ensemble, wl["cout"]
+    g = torch.Generator(device=dev).manual_seed(1)
+    with torch.no_grad():  # per-kernel timing of one eager denoiser call at this batch (also the warm-up)
+        x = torch.randn(B, S, wl["cin"], generator=g, device=dev)
+        t = torch.rand(B, generator=g, device=dev) * (math.pi / 2)
+        model(x, t)
+        pkg.ops.profile_begin()
+        model(x, t)
+        rec = pkg.ops.profile_end()
+        del x
+    smp = pkg.TrigFlowSampler(model, n_steps=args.sampler_steps, device=dev)
+    state0 = torch.randn(B, S, C, generator=g, device=dev)
+    smp.capture(state0, torch.randn(B, S, C, generator=g, device=dev), warmup=1)
+    nfe = 2 * args.sampler_steps - 1
+    for _ in range(args.warmup):
+        smp.rollout(state0, 1, g, use_graph=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    states = smp.rollout(state0, args.steps, g, use_graph=True)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    finite = all(bool(torch.isfinite(s_).all()) for s_ in states)
+    agg = {}
+    for tag, work, unit, ms in rec:
+        a = agg.setdefault(tag, {"launches": 0, "work": 0.0, "ms": 0.0, "unit": unit})
+        a["launches"] += 1; a["work"] += work; a["ms"] += ms
+    dom_tag = max((t_ for t_ in agg if t_.startswith("gemm_256x256")), key=lambda t_: agg[t_]["ms"])
+    dom = agg[dom_tag]
+    tfl = dom["work"] / (dom["ms"] * 1e-3) / 1e12
+    result = {
+        "metric": "denoise steps/s + window-attn MFMA util, 720x1440 grid bf16, 1 GPU",
+        "value": B * nfe * args.steps / elapsed, "unit": "denoise steps/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "forecast_steps_per_s": args.steps / elapsed,
+        "config": {"workload": wl["desc"], "tokens": S, "batch": B, "sampler_steps": args.sampler_steps,
+                   "denoiser_calls_per_forecast_step": nfe, "step": "one forecast step",
+                   "value_counts": "one denoiser call on one member = one denoise step"},
+        "roofline": {"kernel": dom_tag, "bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tfl / PEAK_BF16_TFLOPS, "traffic": None, "flop_per_launch": dom["work"] / dom["launches"],
+                     "avg_launch_ms": dom["ms"] / dom["launches"]},
+        "cpu_baseline": None, "output_finite": finite,
+    }
+    print(json.dumps(result))
 
 
 def cpu_baseline(torch, wl, rows, seconds_cap=60.0):
@@ -103,6 +158,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--ensemble", type=int, default=4, help="config4: ensemble members (batch)")
+    ap.add_argument("--sampler-steps", type=int, default=10, help="config4: sampler steps (2n-1 denoiser calls per forecast step)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the whole grid on ONE GPU; --gpus N > 1 is not supported "
@@ -124,6 +181,10 @@ def main():
     g = torch.Generator(device=dev).manual_seed(1)
     x = torch.randn(1, S, wl["cin"], generator=g, device=dev)
     t = (torch.rand(1, generator=g, device=dev) * (math.pi / 2))
+
+    if wl.get("rollout"):
+        run_rollout(args, pkg, torch, wl, model, dev)
+        return
 
     if args.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB read + 1 GiB written

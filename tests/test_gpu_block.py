@@ -191,3 +191,24 @@ def test_full_grid_block_against_oracle_strips(pkg, cuda, name, geo):
             got = grid_out[rows.to(cuda)].float().cpu()
             err = rel_l2(got, ref)
             assert err <= 1e-2, (name, shifted, k, err)
+
+
+def test_full_grid_ensemble_batch_matches_single_members(pkg, cuda):
+    """configs[4] shape: 4 ensemble members as batch 4 on the 720x1440 grid (4 147 200 rows through every kernel,
+    per-member modulation vectors).  A member's rows of the batched result must be bit-identical to running that
+    member alone: windows, GEMM tiles (1 036 800 = 4050 x 256 rows per member) and norm rows never mix members."""
+    H, W, ws = 720, 1440, 16
+    cfg = OracleConfig.spec(window_size=(ws, ws), image_shape=(H, W), mod_ways=2, dim=1536, heads=24, head_dim=64,
+                            mlp_dim=6144)
+    sd = oracle.init_block_weights(cfg, 23, nontrivial=True)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.randn(4, H * W, cfg.dim, generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    t = torch.randn(4, cfg.dim, generator=torch.Generator().manual_seed(10)).to(cuda)
+    for shifted in (False, True):
+        layer = make_layer(pkg, cfg, sd, cuda, shifted)
+        out = layer(x, t).clone()
+        for b in (0, 3):
+            single = layer(x[b:b + 1].contiguous(), t[b:b + 1].contiguous())
+            torch.cuda.synchronize()
+            assert torch.equal(out[b:b + 1], single), (shifted, b)
+        assert bool(torch.isfinite(out.float()).all())

@@ -47,23 +47,23 @@ __device__ __forceinline__ float erf_poly(float x) {
 }
 __device__ __forceinline__ float gelu_erf_f(float x) { return 0.5f * x * (1.0f + erf_poly(x * 0.70710678118654752440f)); }
 
-// erf-GELU for results that are rounded to bf16: erf(u) = t * P(t^2), t = clamp(u, -3, 3), P a degree-8 minimax
-// polynomial (|error| <= 3.1e-5 in erf, <= 1.6e-5 relative in GELU: 1/100 of a bf16 ulp).  14 VALU operations and no
-// transcendental, against about 24 op-equivalents for the 1.5e-7 version above; the GEMM epilogue is VALU-bound.
+// erf-GELU for results that are rounded to bf16: GELU(x) = x * (0.5 + t * P(t^2)), t = clamp(x, -3 sqrt2, 3 sqrt2),
+// t * P(t^2) = erf(t / sqrt2) / 2 with P a degree-8 minimax polynomial (the 1/sqrt2 and the 1/2 are folded into its
+// coefficients; |error| <= 3.1e-5 in erf, <= 7e-5 absolute in GELU, 1.6e-5 of |x|: 1/100 of a bf16 ulp).  12 VALU
+// operations and no transcendental, against about 24 op-equivalents for the 1.5e-7 version above; the GEMM
+// epilogue is VALU-bound.
 __device__ __forceinline__ float gelu_bf16_f(float x) {
-  const float u = x * 0.70710678118654752440f;
-  const float t = __builtin_amdgcn_fmed3f(u, -3.0f, 3.0f);
+  const float t = __builtin_amdgcn_fmed3f(x, -4.2426406871f, 4.2426406871f);
   const float s = t * t;
-  float p = fmaf(4.074150084e-08f, s, -1.944801170e-06f);
-  p = fmaf(p, s, 4.106021152e-05f);
-  p = fmaf(p, s, -5.110344500e-04f);
-  p = fmaf(p, s, 4.235417116e-03f);
-  p = fmaf(p, s, -2.510283515e-02f);
-  p = fmaf(p, s, 1.110793054e-01f);
-  p = fmaf(p, s, -3.753148615e-01f);
-  p = fmaf(p, s, 1.128268480e+00f);
-  const float hx = 0.5f * x;
-  return fmaf(hx, t * p, hx);
+  float p = fmaf(5.626678031e-11f, s, -5.371805060e-09f);
+  p = fmaf(p, s, 2.268277656e-07f);
+  p = fmaf(p, s, -5.646186328e-06f);
+  p = fmaf(p, s, 9.359038012e-05f);
+  p = fmaf(p, s, -1.109399060e-03f);
+  p = fmaf(p, s, 9.818116262e-03f);
+  p = fmaf(p, s, -6.634692091e-02f);
+  p = fmaf(p, s, 3.989031466e-01f);
+  return x * fmaf(t, p, 0.5f);
 }
 
 }  // namespace aeris

@@ -69,8 +69,17 @@ def run_rollout(args, pkg, torch, wl, model, dev):
     """configs[4]: `--steps` autoregressive forecast steps (a step = one forecast step = 2n-1 denoiser calls on a
     batch of `--ensemble` members), the sampler loop replayed as a HIP graph.  No cpu_baseline leg (N/A: minutes of
     GPU time per step); the roofline object is the dominant GEMM of one eager denoiser call at this batch."""
+    import threading
     H, W = wl["image_shape"]
     S, B, C = H * W, args.ensemble, wl["cout"]
+    done = threading.Event()
+
+    def heartbeat():  # a forecast step is minutes of GPU time with nothing to print; say that the run is alive
+        t_start = time.perf_counter()
+        while not done.wait(45.0):
+            print(f"bench.py: rollout running, {time.perf_counter() - t_start:.0f} s", file=sys.stderr, flush=True)
+
+    threading.Thread(target=heartbeat, daemon=True).start()
     g = torch.Generator(device=dev).manual_seed(1)
     with torch.no_grad():  # per-kernel timing of one eager denoiser call at this batch (also the warm-up)
         x = torch.randn(B, S, wl["cin"], generator=g, device=dev)
@@ -92,6 +101,7 @@ def run_rollout(args, pkg, torch, wl, model, dev):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     finite = all(bool(torch.isfinite(s_).all()) for s_ in states)
+    done.set()
     agg = {}
     for tag, work, unit, ms in rec:
         a = agg.setdefault(tag, {"launches": 0, "work": 0.0, "ms": 0.0, "unit": unit})

@@ -203,8 +203,23 @@ int aeris_embed_prepare_fwd(const float* x, const float* ape, void* out, int64_t
   if (M <= 0 || C <= 0 || K_pad < C || K_pad % 64) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: need M > 0, 0 < C <= K_pad, K_pad %% 64 == 0");
   if (ape && M_ape <= 0) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: M_ape must be positive when ape is given");
   if (!aligned16(out)) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: out must be 16-byte aligned");
-  hipError_t e = aeris::embed_prepare_launch(x, ape, out, M, M_ape > 0 ? M_ape : 1, C, K_pad, reinterpret_cast<hipStream_t>(stream));
+  hipError_t e = aeris::embed_prepare_launch(x, C, 1.0f, nullptr, 0, ape, out, M, M_ape > 0 ? M_ape : 1, K_pad,
+                                             reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_embed_prepare_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_embed_concat_fwd(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
+                           int64_t M, int64_t M_ape, int K_pad, void* stream) {
+  if (!x0 || !x1 || !out) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: x0/x1/out is NULL");
+  if (M <= 0 || C0 <= 0 || C1 <= 0 || K_pad < C0 + C1 || K_pad % 64)
+    return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: need M > 0, C0 > 0, C1 > 0, C0 + C1 <= K_pad, K_pad %% 64 == 0");
+  if (!(div0 != 0.0f)) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: div0 must be non-zero");
+  if (ape && M_ape <= 0) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: M_ape must be positive when ape is given");
+  if (!aligned16(out)) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: out must be 16-byte aligned");
+  hipError_t e = aeris::embed_prepare_launch(x0, C0, div0, x1, C1, ape, out, M, M_ape > 0 ? M_ape : 1, K_pad,
+                                             reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_embed_concat_fwd launch");
   return AERIS_OK;
 }
 

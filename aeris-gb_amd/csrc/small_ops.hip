@@ -87,32 +87,39 @@ hipError_t timestep_embedding_launch(const float* t, float* emb, int B, int dim,
 }
 
 // out[m, k] = bf16(x[m, k] + ape[m % M_ape, k]) for k < C, 0 for C <= k < K_pad.  One thread per 8 output columns.
-__global__ void __launch_bounds__(256) embed_prepare_kernel(const float* __restrict__ x, const float* __restrict__ ape,
-                                                           uint16_t* __restrict__ out, int64_t M, int64_t M_ape, int C,
-                                                           int K_pad) {
+// out[m, :] = [x0[m, :] / div0 | x1[m, :]] + ape[m % M_ape, :], zero padded to K_pad columns (x1 may be absent)
+__global__ void __launch_bounds__(256) embed_prepare_kernel(const float* __restrict__ x0, int C0, float div0,
+                                                           const float* __restrict__ x1, int C1,
+                                                           const float* __restrict__ ape, uint16_t* __restrict__ out,
+                                                           int64_t M, int64_t M_ape, int K_pad) {
   const int cpr = K_pad / 8;
+  const int C = C0 + C1;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= M * cpr) return;
   const int64_t m = i / cpr;
   const int k0 = (int)(i - m * cpr) * 8;
-  const float* xr = x + m * C;
+  const float* r0 = x0 + m * C0;
+  const float* r1 = x1 ? x1 + m * C1 : nullptr;
   const float* ar = ape ? ape + (m % M_ape) * C : nullptr;
   float v[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int k = k0 + e;
     v[e] = 0.f;
-    if (k < C) v[e] = xr[k] + (ar ? ar[k] : 0.f);
+    if (k < C) {
+      const float xv = k < C0 ? (div0 == 1.0f ? r0[k] : r0[k] / div0) : r1[k - C0];
+      v[e] = xv + (ar ? ar[k] : 0.f);
+    }
   }
   u32x4 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
   *reinterpret_cast<u32x4*>(out + m * K_pad + k0) = w;
 }
 
-hipError_t embed_prepare_launch(const float* x, const float* ape, void* out, int64_t M, int64_t M_ape, int C, int K_pad,
-                                hipStream_t stream) {
+hipError_t embed_prepare_launch(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
+                                int64_t M, int64_t M_ape, int K_pad, hipStream_t stream) {
   const int64_t n = M * (K_pad / 8);
-  hipLaunchKernelGGL(embed_prepare_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, ape,
-                     reinterpret_cast<uint16_t*>(out), M, M_ape, C, K_pad);
+  hipLaunchKernelGGL(embed_prepare_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x0, C0, div0, x1, C1,
+                     ape, reinterpret_cast<uint16_t*>(out), M, M_ape, K_pad);
   return hipGetLastError();
 }
 

@@ -343,15 +343,25 @@ class InputStage(nn.Module):
             self._wcache = (key, wp, self.proj.bias.detach().to(torch.bfloat16).contiguous(), k_pad)
         return self._wcache[1:]
 
-    def forward(self, x, interval, out_dtype=None):
+    def forward(self, x, interval, out_dtype=None, cond=None, x_div=1.0):
+        """x [b, n, Cin]; or x [b, n, C0] with cond [b, n, Cin - C0]: the embedding of cat([x / x_div, cond], 2)
+        (inference.py:160) without building the concatenated tensor."""
         b, n, c = x.shape
+        if cond is not None:
+            c += cond.shape[-1]
+        if c != self.model_in_channels:
+            raise ValueError(f"input has {c} channels, the model embeds {self.model_in_channels}")
         ape = self.ape_generated
         if ape is not None:
             ape = ape.reshape(-1, c)
             if ape.shape[0] != n:
                 raise ValueError(f"ape_generated covers {ape.shape[0]} tokens, input has {n}")
         wp, bias, k_pad = self._weights()
-        a = ops.embed_prepare(x.reshape(b * n, c).float().contiguous(), ape, k_pad)
+        if cond is None:
+            a = ops.embed_prepare(x.reshape(b * n, c).float().contiguous(), ape, k_pad)
+        else:
+            a = ops.embed_concat(x.reshape(b * n, -1).float().contiguous(), x_div,
+                                 cond.reshape(b * n, -1).float().contiguous(), ape, k_pad)
         tok = ops.gemm(a, wp, bias, out_dtype=out_dtype or self.model_dtype).view(b, n, -1)
         t = timestep_embedding(interval, tok.shape[-1], self.sinusoidal_emb_max_period)
         return tok, t
@@ -427,8 +437,9 @@ class LocalAERIS(nn.Module):
         self.input_stage.ape_generated = pe.permute(0, 2, 3, 1).reshape(1, H * W, c).contiguous()
         return self.input_stage.ape_generated
 
-    def forward(self, x, dt, return_hidden=False):
-        tok, t = self.input_stage(x, dt, out_dtype=self.residual_dtype)
+    def forward(self, x, dt, return_hidden=False, cond=None, x_div=1.0):
+        """``cond`` / ``x_div``: see InputStage.forward (the sampler's concatenation folded into the embedding)."""
+        tok, t = self.input_stage(x, dt, out_dtype=self.residual_dtype, cond=cond, x_div=x_div)
         half = (self.window_size[0] // 2, self.window_size[1] // 2)
         spare = None
         for i, layer in enumerate(self.layers):

@@ -278,3 +278,25 @@ def embed_prepare(x: torch.Tensor, ape: Optional[torch.Tensor], k_pad: int, out:
         out = torch.empty(M, k_pad, dtype=torch.bfloat16, device=x.device)
     L.call("aeris_embed_prepare_fwd", x.data_ptr(), _ptr(ape), out.data_ptr(), M, m_ape, C, k_pad, _stream())
     return out
+
+
+def embed_concat(x0: torch.Tensor, div0: float, x1: torch.Tensor, ape: Optional[torch.Tensor], k_pad: int,
+                 out: Optional[torch.Tensor] = None):
+    """bf16 [M, k_pad] = [x0 f32 [M, C0] / div0 | x1 f32 [M, C1]] (+ ape f32 [M_ape, C0 + C1]), zero padded."""
+    _dev(x0, "x0", torch.float32)
+    _dev(x1, "x1", torch.float32)
+    C0, C1 = x0.shape[-1], x1.shape[-1]
+    M = x0.numel() // C0
+    if x1.numel() // C1 != M:
+        raise RuntimeError("x0 and x1 must have the same number of rows")
+    m_ape = 0
+    if ape is not None:
+        _dev(ape, "ape", torch.float32)
+        m_ape = ape.numel() // (C0 + C1)
+        if ape.shape[-1] != C0 + C1 or M % m_ape:
+            raise RuntimeError("ape must be [M_ape, C0 + C1] with M a multiple of M_ape")
+    if out is None:
+        out = torch.empty(M, k_pad, dtype=torch.bfloat16, device=x0.device)
+    L.call("aeris_embed_concat_fwd", x0.data_ptr(), C0, float(div0), x1.data_ptr(), C1, _ptr(ape), out.data_ptr(), M,
+           m_ape, k_pad, _stream())
+    return out

@@ -30,8 +30,9 @@ class TrigFlowSampler:
         self._graph = None
 
     def _denoise(self, x, cond, t):
-        # the condition channels follow the state channels (inference.py:160)
-        return self.model(torch.cat([x / self.sigma_data, cond], dim=2), t)
+        # the condition channels follow the state channels (inference.py:160); the division by sigma_data and the
+        # concatenation happen inside the embedding's operand preparation
+        return self.model(x, t, cond=cond, x_div=self.sigma_data)
 
     @torch.no_grad()
     def sample(self, cond: torch.Tensor, latents: torch.Tensor) -> torch.Tensor:

@@ -123,6 +123,13 @@ int aeris_timestep_embedding_fwd(const float* t, float* emb, int B, int dim, flo
 int aeris_embed_prepare_fwd(const float* x, const float* ape, void* out, int64_t M, int64_t M_ape, int C,
                             int K_pad, void* stream);
 
+/* The same with the sampler's channel concatenation folded in: out bf16 [M, K_pad] =
+ * ([x0 f32 [M, C0] / div0 | x1 f32 [M, C1]] + ape f32 [M_ape, C0 + C1] or NULL), zero padded.  x0 is the noised state
+ * (divided by sigma_data), x1 the conditioning channels: torch.cat([x_t / sigma_d, conditioning], dim=2) of
+ * inference.py:160 followed by model.py:350-352, without materialising the concatenated tensor. */
+int aeris_embed_concat_fwd(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
+                           int64_t M, int64_t M_ape, int K_pad, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -281,3 +281,20 @@ def test_embed_prepare_parity(pkg, cuda):
     out = pkg.ops.embed_prepare(x.to(cuda), None, 192).cpu()
     ref[:, :C] = x
     assert torch.equal(out, ref.to(torch.bfloat16))
+
+
+def test_embed_concat_equals_cat_then_prepare(pkg, cuda):
+    """The sampler's cat([x_t / sigma_d, conditioning], 2) (inference.py:160) folded into the operand preparation
+    is bit-identical to concatenating first."""
+    g = torch.Generator().manual_seed(3)
+    B, S, C0, C1 = 2, 300, 69, 69
+    x0, x1, ape = torch.randn(B * S, C0, generator=g), torch.randn(B * S, C1, generator=g), torch.randn(S, C0 + C1, generator=g)
+    for div0 in (1.0, 0.5, 1.7):
+        for a in (ape, None):
+            ref = pkg.ops.embed_prepare(torch.cat([x0 / div0, x1], dim=1).to(cuda), None if a is None else a.to(cuda), 192)
+            got = pkg.ops.embed_concat(x0.to(cuda), div0, x1.to(cuda), None if a is None else a.to(cuda), 192)
+            assert torch.equal(got, ref), (div0, a is None)
+    # uneven split
+    got = pkg.ops.embed_concat(x0[:, :5].contiguous().to(cuda), 2.0, x1.to(cuda), None, 128)
+    ref = pkg.ops.embed_prepare(torch.cat([x0[:, :5] / 2.0, x1], dim=1).to(cuda), None, 128)
+    assert torch.equal(got, ref)

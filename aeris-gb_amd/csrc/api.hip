@@ -30,6 +30,7 @@ int ensure_init() {
   std::call_once(g_init_once, [] {
     g_init_status = aeris::gemm_configure_all();
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_configure_all();
+    if (g_init_status == hipSuccess) g_init_status = aeris::attention_stream_configure_all();
   });
   if (g_init_status != hipSuccess) return hip_fail(g_init_status, "aeris_init (hipFuncSetAttribute)");
   return AERIS_OK;
@@ -119,13 +120,23 @@ int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_tabl
   if (heads <= 0 || head_dim <= 0) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: heads/head_dim must be positive");
   if (int rc = check_window_geometry(B, H, W, ws_y, ws_x, shift_y, shift_x)) return rc;
   if (!(scale > 0.f)) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: scale must be positive");
-  if (!aeris::attention_supported(ws_y, ws_x, head_dim))
+  const bool small = aeris::attention_supported(ws_y, ws_x, head_dim);
+  const bool masked = use_mask && (shift_y > 0 || shift_x > 0);
+  if (!small && !aeris::attention_stream_supported(ws_y, ws_x, head_dim, bias_table != nullptr, masked))
     return fail(AERIS_EUNSUPPORTED,
-                "aeris_window_attention_fwd: no kernel for window %dx%d head_dim %d (built: 8x8, 12x12, 16x16 with head_dim 32 or 64)",
-                ws_y, ws_x, head_dim);
-  if ((int64_t)B * (H / ws_y) * (W / ws_x) * heads > 0x7fffffffLL)
-    return fail(AERIS_EUNSUPPORTED, "aeris_window_attention_fwd: more than 2^31-1 (window, head) pairs");
+                "aeris_window_attention_fwd: no kernel for window %dx%d head_dim %d%s (built: 8x8, 12x12, 16x16 with head_dim "
+                "32 or 64, bias and mask optional; any window of up to 4096 tokens with head_dim 64 or 128 without bias and mask)",
+                ws_y, ws_x, head_dim, bias_table ? " with a bias table" : (masked ? " with the shift mask" : ""));
+  const int64_t units = (int64_t)B * (H / ws_y) * (W / ws_x) * heads;
+  if (units > 0x7fffffffLL || (!small && (units + 8) * (((int64_t)ws_y * ws_x + 127) / 128) > 0x7fffffffLL))
+    return fail(AERIS_EUNSUPPORTED, "aeris_window_attention_fwd: more than 2^31-1 workgroups");
   if (int rc = ensure_init()) return rc;
+  if (!small) {
+    hipError_t e = aeris::attention_stream_launch(qkv, out, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x, scale,
+                                                  reinterpret_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "aeris_window_attention_fwd launch (streaming kernel)");
+    return AERIS_OK;
+  }
   hipError_t e = aeris::attention_launch(qkv, out, bias_table, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x,
                                          use_mask, scale, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_window_attention_fwd launch");

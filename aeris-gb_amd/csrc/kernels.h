@@ -16,6 +16,11 @@ hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, 
 
 // returns hipErrorInvalidValue when (ws_y, ws_x, head_dim) has no instantiation
 bool attention_supported(int ws_y, int ws_x, int head_dim);
+// streaming kernel (window_attention_stream.hip): any window of up to 4096 tokens, head_dim 64 / 128, no bias, no mask
+bool attention_stream_supported(int ws_y, int ws_x, int head_dim, bool has_bias, bool use_mask);
+hipError_t attention_stream_configure_all();
+hipError_t attention_stream_launch(const void* qkv, void* out, int B, int H, int W, int heads, int head_dim, int ws_y,
+                                   int ws_x, int shift_y, int shift_x, float scale, hipStream_t stream);
 hipError_t attention_launch(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
                             int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
                             hipStream_t stream);

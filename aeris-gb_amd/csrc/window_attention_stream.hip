@@ -1,0 +1,311 @@
+// Windowed multi-head self-attention for gfx950, streaming variant: windows of any size up to 4096 tokens
+// (the reference's 60 x 60) and head_dim 64 or 128, no relative-position bias, no shift mask (model.py:289-293).
+//
+// One workgroup = 128 queries of one (window, head): 4 waves x 32 queries.  The keys of the window are streamed
+// through LDS in chunks of 64 (double buffered: the global loads of chunk j+1 are in flight while chunk j is
+// being consumed) with an online softmax (running row max m and row sum l, output rescaled only when a max
+// moves).  Window partition, window reverse and the cyclic shift are address arithmetic exactly as in the
+// one-window-per-workgroup kernel (window_attention.hip); the token row of every window position is computed once
+// per workgroup into an LDS table, so the streaming loop needs no integer division.
+//
+//   K chunk [64][HD]   global -> registers -> LDS, 16-byte chunks XOR-swizzled (conflict-free ds_read_b128)
+//   V chunk [64][HD]   global -> registers (4 keys x 8 d per thread) -> 4x8 register transpose -> LDS as
+//                      V^T [HD][64], key groups permuted so that a PV fragment is one ds_read_b128
+//   Q                  global -> registers (MFMA B operand), once
+//   S^T = K Q^T        v_mfma_f32_32x32x16_bf16; lane = one query, registers = keys
+//   O^T += V^T P^T     P^T straight from the S^T accumulator registers
+// The query blocks of one (window, head) are placed on the same XCD (blockIdx % 8), so its K / V rows are fetched
+// into that XCD's L2 once and re-read from there by the other query blocks.
+#include "common.h"
+#include "kernels.h"
+
+namespace aeris {
+
+namespace {
+
+struct StreamParams {
+  const uint16_t* qkv;
+  uint16_t* out;
+  int B, H, W, heads;
+  int nWy, nWx, ws_y, ws_x;
+  int sy, sx;
+  int n_units, qblks;
+  float scale;
+};
+
+constexpr int KC = 64;    // keys per chunk
+constexpr int QB = 128;   // queries per workgroup
+constexpr int MAX_L = 4096;
+
+// byte offset of 16-byte chunk `chunk` of row `row` in a tile with 128-byte rows (8 chunks), swizzled over double rows
+__device__ __forceinline__ uint32_t off128(int row, int chunk) {
+  return (uint32_t)((row >> 1) * 256 + (((((row & 1) << 3) | chunk) ^ ((row >> 1) & 7)) << 4));
+}
+// the same for 256-byte rows (16 chunks)
+__device__ __forceinline__ uint32_t off256(int row, int chunk) { return (uint32_t)(row * 256 + ((chunk ^ (row & 15)) << 4)); }
+
+template <int HD>
+struct StreamCfg {
+  static constexpr int K_BYTES = KC * HD * 2;
+  static constexpr int V_BYTES = HD * KC * 2;
+  static constexpr int BUF = K_BYTES + V_BYTES;
+  static constexpr int TBL_OFF = 2 * BUF;
+};
+
+}  // namespace
+
+template <int HD>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+window_attention_stream_kernel(StreamParams p) {
+  using Cfg = StreamCfg<HD>;
+  constexpr int CH = HD / 8;   // 16-byte chunks per head row
+  constexpr int KS = HD / 16;  // k16 steps of QK^T
+  constexpr int DB = HD / 32;  // 32-row blocks of O^T
+  constexpr int NT = 256;
+  constexpr int KIT = KC * CH / NT;                     // 16-byte K pieces per thread and chunk (2 or 4)
+  constexpr int V_ITEMS = (KC / 4) * CH;                // (4 keys x 8 d) V pieces per chunk: 128 or 256
+  constexpr float LOG2E = 1.4426950408889634f;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  int* tok = reinterpret_cast<int*>(smem + Cfg::TBL_OFF);  // token row (inside the image) of every window position
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l31 = lane & 31, hi = lane >> 5;
+
+  // all query blocks of one (window, head) on one XCD
+  const int xcd = blockIdx.x & 7, s_idx = blockIdx.x >> 3;
+  const int unit = xcd + 8 * (s_idx / p.qblks);
+  const int qb = s_idx % p.qblks;
+  if (unit >= p.n_units) return;
+  const int head = unit % p.heads;
+  const int win = unit / p.heads;
+  const int wpi = p.nWy * p.nWx;
+  const int b = win / wpi;
+  const int wrem = win - b * wpi;
+  const int wy = wrem / p.nWx, wx = wrem - wy * p.nWx;
+  const int H = p.H, W = p.W;
+  const int L = p.ws_y * p.ws_x;
+  const int inner = p.heads * HD;
+  const int64_t ld_qkv = 3 * (int64_t)inner;
+  const int64_t img_base = (int64_t)b * H * W;
+  const int y0 = wy * p.ws_y + p.sy, x0 = wx * p.ws_x + p.sx;
+
+  for (int pos = tid; pos < L; pos += NT) {
+    int Y = y0 + pos / p.ws_x;
+    int X = x0 + pos % p.ws_x;
+    if (Y >= H) Y -= H;
+    if (X >= W) X -= W;
+    tok[pos] = Y * W + X;
+  }
+  __syncthreads();
+
+  // ---- Q fragments (B operand): lane = query, 8 consecutive d per k16 step
+  int qpos = qb * QB + wave * 32 + l31;
+  const bool q_valid = qpos < L;
+  if (!q_valid) qpos = L - 1;
+  const int64_t q_row = img_base + tok[qpos];
+  bf16x8 qf[KS];
+  {
+    const uint16_t* qp = p.qkv + q_row * ld_qkv + head * HD + hi * 8;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
+  }
+
+  const uint16_t* kbase = p.qkv + img_base * ld_qkv + inner + head * HD;
+  const uint16_t* vbase = p.qkv + img_base * ld_qkv + 2 * inner + head * HD;
+  const int nch = (L + KC - 1) / KC;
+
+  u32x4 kreg[KIT], vreg[4];
+  const bool v_item = (V_ITEMS >= NT) || tid < V_ITEMS;  // head_dim 64: half of the threads carry a V piece
+  auto load_chunk = [&](int j) {
+    const int key0 = j * KC;
+#pragma unroll
+    for (int it = 0; it < KIT; ++it) {
+      const int idx = tid + it * NT, key = idx / CH, c = idx % CH;
+      int kp = key0 + key;
+      if (kp > L - 1) kp = L - 1;  // rows past the window: any valid row, their scores are masked
+      kreg[it] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)tok[kp] * ld_qkv + c * 8);
+    }
+    if (v_item) {
+      const int kg = tid / CH, c = tid % CH;
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        int kp = key0 + kg * 4 + jj;
+        if (kp > L - 1) kp = L - 1;
+        vreg[jj] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)tok[kp] * ld_qkv + c * 8);
+      }
+    }
+  };
+  auto store_chunk = [&](int buf) {
+    unsigned char* sK = smem + buf * Cfg::BUF;
+    unsigned char* sV = sK + Cfg::K_BYTES;
+#pragma unroll
+    for (int it = 0; it < KIT; ++it) {
+      const int idx = tid + it * NT, key = idx / CH, c = idx % CH;
+      *reinterpret_cast<u32x4*>(sK + (HD == 64 ? off128(key, c) : off256(key, c))) = kreg[it];
+    }
+    // V: 4 keys x 8 d register transpose -> V^T[d][key].  Inside every block of 16 keys the four key groups are
+    // stored in the order 0, 2, 1, 3: the 8 keys one lane needs for a k16 step of PV (4hi..4hi+3 and
+    // 8+4hi..8+4hi+3, the accumulator layout of S^T) are then one aligned 16-byte chunk.
+    if (v_item) {
+      const int kg = tid / CH, c = tid % CH;
+      const int pos = (kg & ~3) | (((kg & 1) << 1) | ((kg >> 1) & 1));
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {  // word w holds d = 8c + 2w (low half) and 8c + 2w + 1 (high half)
+        u32x2 lo, hi2;
+        lo.x = (vreg[0][w] & 0xffffu) | (vreg[1][w] << 16);
+        lo.y = (vreg[2][w] & 0xffffu) | (vreg[3][w] << 16);
+        hi2.x = (vreg[0][w] >> 16) | (vreg[1][w] & 0xffff0000u);
+        hi2.y = (vreg[2][w] >> 16) | (vreg[3][w] & 0xffff0000u);
+        const int d0 = c * 8 + 2 * w, d1 = d0 + 1;
+        *reinterpret_cast<u32x2*>(sV + off128(d0, pos >> 1) + (pos & 1) * 8) = lo;
+        *reinterpret_cast<u32x2*>(sV + off128(d1, pos >> 1) + (pos & 1) * 8) = hi2;
+      }
+    }
+  };
+
+  const float c = p.scale * LOG2E;
+  float m = -INFINITY, l = 0.f;
+  f32x16 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+
+  load_chunk(0);
+  store_chunk(0);
+  __syncthreads();
+
+  for (int j = 0; j < nch; ++j) {
+    if (j + 1 < nch) load_chunk(j + 1);
+    const unsigned char* sK = smem + (j & 1) * Cfg::BUF;
+    const unsigned char* sV = sK + Cfg::K_BYTES;
+
+    // ---- S^T = K Q^T for the 64 keys of the chunk: acc[kb][4g+i] = <k[key], q>, key = 64j + 32kb + 8g + 4hi + i
+    f32x16 acc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[kb][e] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int row = kb * 32 + l31, ch = s * 2 + hi;
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + (HD == 64 ? off128(row, ch) : off256(row, ch)));
+        acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], acc[kb], 0, 0, 0);
+      }
+    }
+    if (j * KC + KC > L) {  // last, partial chunk (uniform): keys past the window do not take part
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = j * KC + kb * 32 + (e >> 2) * 8 + hi * 4 + (e & 3);
+          if (key >= L) acc[kb][e] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax (exp2 domain): new row max, rescale what has been accumulated if any max moved
+    float cm = acc[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) cm = fmaxf(fmaxf(cm, acc[kb][e]), acc[kb][e + 1]);
+    cm *= c;
+    cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+    const float m_new = fmaxf(m, cm);
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // 0 for the first chunk (m = -inf)
+      l *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+      m = m_new;
+    }
+    uint32_t pk[2][8];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int h2 = 0; h2 < 8; ++h2) {
+        const float e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -m));
+        const float e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -m));
+        l += e0 + e1;
+        pk[kb][h2] = pack_bf16x2(e0, e1);
+      }
+
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        // k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one V^T chunk
+        const u32x4 pw = {pk[kb][4 * t2], pk[kb][4 * t2 + 1], pk[kb][4 * t2 + 2], pk[kb][4 * t2 + 3]};
+        const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+        const int ch = kb * 4 + t2 * 2 + hi;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(sV + off128(db * 32 + l31, ch));
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, o[db], 0, 0, 0);
+        }
+      }
+
+    if (j + 1 < nch) store_chunk((j + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i]
+  l += __shfl_xor(l, 32, 64);
+  const float inv = __builtin_amdgcn_rcpf(l);
+  if (q_valid) {
+    uint16_t* op = p.out + q_row * inner + head * HD + hi * 4;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w2;
+        w2.x = pack_bf16x2(o[db][g * 4] * inv, o[db][g * 4 + 1] * inv);
+        w2.y = pack_bf16x2(o[db][g * 4 + 2] * inv, o[db][g * 4 + 3] * inv);
+        *reinterpret_cast<u32x2*>(op + db * 32 + g * 8) = w2;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+
+static int stream_smem(int head_dim, int L) { return 2 * (KC * head_dim * 2 + head_dim * KC * 2) + ((L * 4 + 15) / 16) * 16; }
+
+bool attention_stream_supported(int ws_y, int ws_x, int head_dim, bool has_bias, bool use_mask) {
+  const int64_t L = (int64_t)ws_y * ws_x;
+  return (head_dim == 64 || head_dim == 128) && L >= 1 && L <= MAX_L && !has_bias && !use_mask;
+}
+
+hipError_t attention_stream_configure_all() {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_stream_kernel<64>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, stream_smem(64, MAX_L));
+  if (e != hipSuccess) return e;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_stream_kernel<128>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, stream_smem(128, MAX_L));
+}
+
+hipError_t attention_stream_launch(const void* qkv, void* out, int B, int H, int W, int heads, int head_dim, int ws_y,
+                                   int ws_x, int shift_y, int shift_x, float scale, hipStream_t stream) {
+  StreamParams p;
+  p.qkv = reinterpret_cast<const uint16_t*>(qkv);
+  p.out = reinterpret_cast<uint16_t*>(out);
+  p.B = B; p.H = H; p.W = W; p.heads = heads;
+  p.nWy = H / ws_y; p.nWx = W / ws_x; p.ws_y = ws_y; p.ws_x = ws_x;
+  p.sy = shift_y; p.sx = shift_x;
+  p.scale = scale;
+  const int L = ws_y * ws_x;
+  p.n_units = B * p.nWy * p.nWx * heads;
+  p.qblks = (L + QB - 1) / QB;
+  const int64_t grid = (int64_t)((p.n_units + 7) / 8) * 8 * p.qblks;
+  const int smem = stream_smem(head_dim, L);
+  if (head_dim == 64)
+    hipLaunchKernelGGL(window_attention_stream_kernel<64>, dim3((unsigned)grid), dim3(256), smem, stream, p);
+  else
+    hipLaunchKernelGGL(window_attention_stream_kernel<128>, dim3((unsigned)grid), dim3(256), smem, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace aeris

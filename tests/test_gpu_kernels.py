@@ -125,6 +125,49 @@ def test_window_attention_parity(pkg, cuda, case):
     assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
 
 
+STREAM_CASES = [
+    # B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x  -- shapes only the streaming kernel takes
+    (1, 120, 120, 2, 128, 60, 60, 30, 30),   # the reference's window: 3600 tokens, head_dim 128 (model.py:22-27), shifted
+    (1, 60, 120, 1, 128, 60, 60, 0, 0),
+    (2, 40, 60, 3, 64, 20, 20, 10, 10),      # L = 400: partial last key chunk and query block
+    (1, 32, 32, 2, 128, 16, 16, 8, 8),       # L = 256 with head_dim 128
+    (1, 24, 40, 2, 128, 12, 20, 6, 10),      # rectangular window, L = 240
+    (1, 18, 14, 1, 64, 9, 7, 4, 3),          # L = 63: less than one key chunk, odd sizes
+    (1, 64, 128, 2, 64, 64, 64, 32, 32),     # L = 4096, the largest window
+]
+
+
+@pytest.mark.parametrize("case", STREAM_CASES, ids=lambda c: f"B{c[0]}_{c[1]}x{c[2]}_h{c[3]}x{c[4]}_ws{c[5]}x{c[6]}_s{c[7]}x{c[8]}")
+def test_window_attention_streaming_parity(pkg, cuda, case):
+    """Windows of more than 256 tokens and head_dim 128 (no bias, no mask: what the reference's model.py runs) go
+    through the streaming kernel; same oracle, same tolerance as the one-window-per-workgroup kernel."""
+    B, H, W, heads, hd, wsy, wsx, shy, shx = case
+    g = torch.Generator().manual_seed(H * W + heads)
+    inner = heads * hd
+    qkv = bf(torch.randn(B, H * W, 3 * inner, generator=g))
+    cfg = OracleConfig(dim=inner, heads=heads, head_dim=hd, mlp_dim=inner, window_size=(wsy, wsx), image_shape=(H, W),
+                       rel_pos_bias=False, shift_mask=False)
+    ref = attention_core(cfg, qkv.float(), (shy, shx), None)
+    out = pkg.ops.window_attention(qkv.to(cuda).view(B * H * W, -1), B, (H, W), heads, hd, (wsy, wsx), (shy, shx), None, False)
+    out2 = pkg.ops.window_attention(qkv.to(cuda).view(B * H * W, -1), B, (H, W), heads, hd, (wsy, wsx), (shy, shx), None, False)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    err = rel_l2(out.view(B, H * W, inner), ref)
+    assert err <= 6e-3, err
+    assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
+
+
+def test_window_attention_streaming_rejects_bias_and_mask(pkg, cuda):
+    qkv = torch.zeros(60 * 60, 3 * 128, dtype=torch.bfloat16, device=cuda)
+    table = torch.zeros(119 * 119, 1, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(pkg.AerisError) as e:
+        pkg.ops.window_attention(qkv, 1, (60, 60), 1, 128, (60, 60), (0, 0), table, False)
+    assert e.value.code == -2
+    with pytest.raises(pkg.AerisError) as e:
+        pkg.ops.window_attention(qkv, 1, (60, 60), 1, 128, (60, 60), (30, 30), None, True)
+    assert e.value.code == -2
+
+
 @pytest.mark.parametrize("geo", [(2, 32, 64, 8, 4), (1, 36, 60, 12, 6), (1, 48, 80, 16, 8), (1, 32, 32, 16, 0)])
 @pytest.mark.parametrize("disp", [(0, 0), (0, -1), (1, 0), (-2, 3)])
 def test_attention_index_map_bit_exact(pkg, cuda, geo, disp):

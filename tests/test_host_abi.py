@@ -78,8 +78,12 @@ def test_argument_validation_needs_no_gpu(pkg):
     f = lib.aeris_window_attention_fwd
     assert f(None, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, None) == L.EINVAL
     assert f(p16 + 2, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, None) == L.EINVAL  # misaligned
-    assert f(p16, p16, None, 1, 60, 60, 12, 128, 60, 60, 0, 0, 0, 0.1, None) == L.EUNSUPPORTED  # the reference's 60x60x128
-    assert "no kernel" in L.last_error()
+    # the reference's 60x60 x 128 runs on the streaming kernel, but not with a bias table or the shift mask
+    assert f(p16, p16, p16, 1, 60, 60, 12, 128, 60, 60, 0, 0, 0, 0.1, None) == L.EUNSUPPORTED
+    assert "no kernel" in L.last_error() and "bias" in L.last_error()
+    assert f(p16, p16, None, 1, 60, 60, 12, 128, 60, 60, 30, 30, 1, 0.1, None) == L.EUNSUPPORTED
+    assert f(p16, p16, None, 1, 65, 65, 2, 64, 65, 65, 0, 0, 0, 0.1, None) == L.EUNSUPPORTED  # 4225 tokens per window
+    assert f(p16, p16, None, 1, 16, 16, 2, 96, 16, 16, 0, 0, 0, 0.1, None) == L.EUNSUPPORTED  # head_dim 96
     assert f(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.0, None) == L.EINVAL  # scale
     assert f(p16, p16, None, 1, 16, 20, 2, 64, 16, 16, 0, 0, 0, 0.125, None) == L.EINVAL  # grid not a multiple
     # norm

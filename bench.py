@@ -40,6 +40,10 @@ WORKLOADS = {
                     cin=138, cout=69, rollout=True,
                     desc="configs[4]: ensemble rollout with the configs[3] denoiser, members as batch, Heun ODE sampler "
                          "replayed as one HIP graph per forecast step"),
+    "refwin": dict(image_shape=(720, 1440), dim=1536, heads=12, head_dim=128, window=60, mlp_dim=6144, blocks=24,
+                   cin=138, cout=69, preset="ref",
+                   desc="configs[3] grid and widths with the reference's own block (model.py: RMSNorm, 3-way modulation before "
+                        "the norm, SwiGLU, no biases) and window geometry (60x60 windows of 3600 tokens, 12 heads x 128)"),
     "config1": dict(image_shape=(180, 360), dim=512, heads=8, head_dim=64, window=12, mlp_dim=2048, blocks=2,
                     cin=138, cout=69, desc="configs[1]-shaped denoiser, 180x360 grid, 2 blocks, dim 512, 12x12 windows"),
 }
@@ -50,8 +54,8 @@ def build_model(pkg, torch, wl, device, residual_dtype):
     model = pkg.LocalAERIS(device_mesh=None, heads=wl["heads"], dim=wl["dim"], head_dim=wl["head_dim"],
                            mlp_dim=wl["mlp_dim"], window_size=(ws, ws), image_shape=wl["image_shape"], rope_base=10_000,
                            sublayers=1, sinusoidal_emb_max_period=10_000, n_layers=wl["blocks"] + 2,
-                           model_in_channels=wl["cin"], model_out_channels=wl["cout"], preset="spec", mod_ways=2,
-                           residual_dtype=residual_dtype)
+                           model_in_channels=wl["cin"], model_out_channels=wl["cout"], residual_dtype=residual_dtype,
+                           **(dict(preset="ref") if wl.get("preset") == "ref" else dict(preset="spec", mod_ways=2)))
     model = model.to(device)
     g = torch.Generator(device=device).manual_seed(0)
     with torch.no_grad():
@@ -261,10 +265,12 @@ def main():
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": wl["desc"], "tokens": S, "batch": 1, "residual_stream": args.residual,
-                   "preset": "spec (LayerNorm, scale/shift modulation, rel-pos bias, shift mask, GELU MLP, biases)"},
+                   "preset": ("ref (RMSNorm, shift/scale/gate modulation before the norm, SwiGLU MLP, no biases, bias table or mask)"
+                              if wl.get("preset") == "ref" else
+                              "spec (LayerNorm, scale/shift modulation, rel-pos bias, shift mask, GELU MLP, biases)")},
         "roofline": roofline, "kernels": kernels, "output_finite": finite,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and wl.get("preset") != "ref":  # the CPU leg times the headline block only
         result["cpu_baseline"] = cpu_baseline(torch, wl, args.cpu_rows)
         result["gpu_over_cpu"] = result["value"] / result["cpu_baseline"]["value"]
     print(json.dumps(result))

@@ -119,6 +119,23 @@ def test_small_model_parity(pkg, cuda, preset, res_dt):
     assert rel_l2(out, ref) <= 1e-2
 
 
+def test_reference_window_model_parity(pkg, cuda):
+    """The reference's own window geometry (60 x 60 windows of 3600 tokens, head_dim 128, model.py:22-27; preset
+    "ref": RMSNorm, 3-way modulation, SwiGLU, no bias / mask) on a 120 x 180 grid: input stage -> 2 layers (the
+    second on the half-window-shifted grid) -> output stage, against the oracle."""
+    cfg = OracleConfig.ref(n_layers=4, in_channels=138, out_channels=69, dim=256, heads=2, head_dim=128, mlp_dim=512,
+                           window_size=(60, 60), image_shape=(120, 180))
+    sd = oracle.init_model_weights(cfg, 13, nontrivial=True)
+    model = make_model(pkg, cfg, sd, cuda, torch.bfloat16, "ref")
+    g = torch.Generator().manual_seed(31)
+    x, dt = torch.randn(1, 120 * 180, 138, generator=g), torch.tensor([0.7])
+    ref, ref_h = oracle.model_forward(cfg, sd, x, dt, return_hidden=True)
+    out, hid = model(x.to(cuda), dt.to(cuda), return_hidden=True)
+    torch.cuda.synchronize()
+    assert rel_l2(hid, ref_h) <= 1e-2, rel_l2(hid, ref_h)
+    assert rel_l2(out, ref) <= 1e-2, rel_l2(out, ref)
+
+
 def test_sampler_parity_and_graph_replay(pkg, cuda):
     cfg = OracleConfig.ref(n_layers=4, in_channels=24, out_channels=8, dim=128, heads=2, head_dim=64, mlp_dim=256,
                            window_size=(8, 8), image_shape=(16, 24))

@@ -42,6 +42,12 @@ GEMM_CASES = [
     (3000, 256, 128, "swiglu", False, 0, None, torch.bfloat16),   # small-tile SwiGLU
     (70000, 1024, 256, "swiglu", True, 0, None, torch.bfloat16),  # big-tile SwiGLU
     (500, 100, 64, "swiglu", False, 0, None, torch.float32),      # SwiGLU with ragged N
+    # big tiles whose rows straddle a batch boundary (64 800 rows per batch = 253 tiles + 32 rows): per-lane gate rows
+    (129600, 768, 256, None, True, 2, torch.bfloat16, torch.bfloat16),
+    (129600, 512, 128, None, False, 2, torch.float32, torch.float32),
+    (66000, 1028, 64, None, True, 0, torch.bfloat16, torch.bfloat16),  # big tiles, one k-tile, last 16-byte chunk half inside
+    (70000, 1100, 128, "swiglu", True, 0, None, torch.bfloat16),  # big-tile SwiGLU with ragged N
+    (300, 4096, 192, "gelu", True, 0, torch.bfloat16, torch.bfloat16),  # 2 x 16 big tiles: most workgroups idle or one tile
 ]
 
 

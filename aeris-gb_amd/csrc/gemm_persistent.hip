@@ -281,15 +281,23 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       if (p.res_dtype >= 0) load_res(0);
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
+        // A row's 16-byte chunk c (8 columns) is split between lane l31 (columns 0-3) and lane l31 + 32 (4-7).
+        // v_permlane32_swap on the registers of chunks 2m and 2m+1 gives the lower lane all of chunk 2m and the
+        // upper lane all of chunk 2m+1: one conflict-free ds_write_b128 per lane and chunk pair instead of two
+        // 4-way conflicting ds_write_b64.
+        u32x2 w2[NJ * 4];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
           float v[4][4];
           fragment(i, j, v);
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            u32x2 w2 = {pack_bf16x2(v[g][0], v[g][1]), pack_bf16x2(v[g][2], v[g][3])};
-            *reinterpret_cast<u32x2*>(stg + l31 * 128 + (((j * 4 + g) ^ (l31 & 7)) << 4) + hi * 8) = w2;
-          }
+          for (int g = 0; g < 4; ++g) w2[j * 4 + g] = u32x2{pack_bf16x2(v[g][0], v[g][1]), pack_bf16x2(v[g][2], v[g][3])};
+        }
+#pragma unroll
+        for (int mm = 0; mm < NJ * 2; ++mm) {
+          const auto rx = __builtin_amdgcn_permlane32_swap(w2[2 * mm].x, w2[2 * mm + 1].x, false, false);
+          const auto ry = __builtin_amdgcn_permlane32_swap(w2[2 * mm].y, w2[2 * mm + 1].y, false, false);
+          *reinterpret_cast<u32x4*>(stg + swz_off(l31, 2 * mm + hi)) = u32x4{rx[0], ry[0], rx[1], ry[1]};
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -298,7 +306,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
           const int row = rrow + 8 * it;
-          u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+          u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + swz_off(row, rch));
           if (p.gate || p.res_dtype >= 0) {
             float o[8];
 #pragma unroll
@@ -384,7 +392,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           f32x4 w4 = {v[g][0], v[g][1], v[g][2], v[g][3]};
-          *reinterpret_cast<f32x4*>(stg + l31 * 128 + (((g * 2 + hi) ^ (l31 & 7)) << 4)) = w4;
+          *reinterpret_cast<f32x4*>(stg + swz_off(l31, g * 2 + hi)) = w4;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -393,7 +401,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
           const int row = rrow + 8 * it;
-          f32x4 o = *reinterpret_cast<const f32x4*>(stg + row * 128 + ((rch ^ (row & 7)) << 4));
+          f32x4 o = *reinterpret_cast<const f32x4*>(stg + swz_off(row, rch));
           if (gate_per_lane) {
             int n = unit_col(u);
             if (n >= N) n = N - 4;

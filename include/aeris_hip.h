@@ -83,7 +83,9 @@ int aeris_shift_region_ids(int H, int W, int ws_y, int ws_x, int shift_y, int sh
  *   use_mask != 0 adds the Swin-v1 cyclic-shift mask (-100 across regions) when a shift is non-zero
  * Window partition / reverse and the cyclic shift are folded into the load / store addresses.
  * Replaces model.py:300-307 (+ the swin_shift calls at model.py:471-475 on one device).
- * Supported: ws_y*ws_x <= 256, head_dim in {32, 64}, ws_x % 4 == 0. */
+ * Supported: windows 8x8, 12x12, 16x16 with head_dim 32 or 64 (bias table and mask optional); without bias table and
+ * mask any window of up to 4096 tokens with head_dim 64 or 128, which includes the reference's 60x60 windows and
+ * head_dim 128 (model.py:22-27).  Anything else: AERIS_EUNSUPPORTED. */
 int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_table, int B, int H, int W,
                                int heads, int head_dim, int ws_y, int ws_x, int shift_y, int shift_x,
                                int use_mask, float scale, void* stream);

@@ -26,11 +26,21 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
 
-// 64-lane wavefront reductions
+// 64-lane wavefront sum, the same value in every lane.  Data-parallel-primitive adds inside the 16-lane rows (quad
+// permutes, half mirror, mirror), two row broadcasts across the rows, total read from lane 63: six VALU operations
+// instead of six round trips through the LDS crossbar (ds_bpermute), which a row-per-wave kernel feels twice per row.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {  // v + v[lane selected by CTRL]; rows outside ROW_MASK add 0
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, true));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
+  v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane holds the sum of its row
+  v = dpp_add<0x142, 0xA>(v);  // row_bcast15: rows 1 and 3 add the row before them
+  v = dpp_add<0x143, 0xC>(v);  // row_bcast31: rows 2 and 3 add rows 0 + 1
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }

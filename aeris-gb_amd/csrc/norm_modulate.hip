@@ -32,7 +32,8 @@ struct NormParams {
   float eps;
 };
 
-template <int NV, bool X_F32, bool PRE>
+// FULL: d == NV * 512, every lane holds NV full 16-byte pieces of the row (no per-piece predicates in the loop)
+template <int NV, bool X_F32, bool PRE, bool FULL>
 __global__ void __launch_bounds__(256) norm_modulate_kernel(NormParams p) {
   const int lane = threadIdx.x & 63;
   const int64_t wave_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -45,7 +46,7 @@ __global__ void __launch_bounds__(256) norm_modulate_kernel(NormParams p) {
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
     col[v] = (v * 64 + lane) * 8;
-    act[v] = col[v] < d;
+    act[v] = FULL || col[v] < d;
   }
 
   float G[NV][8], Bc[NV][8], P1[PRE ? NV : 1][8], P0[PRE ? NV : 1][8];
@@ -181,13 +182,19 @@ static hipError_t launch_norm(const NormParams& p, bool x_f32, bool pre, hipStre
   const int64_t cap = 256 * 8;
   if (blocks > cap) blocks = cap;
   dim3 grid((unsigned)blocks), block(256);
+#define AERIS_NORM_GO(XF, PR)                                                                                   \
+  do {                                                                                                          \
+    if (p.d == NV * 512) hipLaunchKernelGGL((norm_modulate_kernel<NV, XF, PR, true>), grid, block, 0, stream, p);  \
+    else hipLaunchKernelGGL((norm_modulate_kernel<NV, XF, PR, false>), grid, block, 0, stream, p);                 \
+  } while (0)
   if (x_f32) {
-    if (pre) hipLaunchKernelGGL((norm_modulate_kernel<NV, true, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((norm_modulate_kernel<NV, true, false>), grid, block, 0, stream, p);
+    if (pre) AERIS_NORM_GO(true, true);
+    else AERIS_NORM_GO(true, false);
   } else {
-    if (pre) hipLaunchKernelGGL((norm_modulate_kernel<NV, false, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((norm_modulate_kernel<NV, false, false>), grid, block, 0, stream, p);
+    if (pre) AERIS_NORM_GO(false, true);
+    else AERIS_NORM_GO(false, false);
   }
+#undef AERIS_NORM_GO
   return hipGetLastError();
 }
 

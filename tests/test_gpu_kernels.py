@@ -110,6 +110,11 @@ ATTN_CASES = [
     (2, 32, 32, 2, 64, 16, 0, False, False),
     (1, 32, 48, 2, 32, 16, 8, False, True),
     (1, 16, 16, 1, 64, 16, 8, True, True),      # one window: every border region in it
+    # more (window, head) units than the chip runs at once (2 workgroups per CU), many heads, an odd head count
+    (1, 160, 160, 24, 64, 16, 8, True, True),   # configs[3] heads: 2400 units
+    (2, 16, 192, 90, 64, 16, 8, True, True),    # 2160 units, 90 heads
+    (1, 64, 96, 90, 64, 16, 0, False, False),   # 2160 units, no bias
+    (1, 48, 720, 17, 64, 16, 8, True, False),   # 2295 units, 17 heads
 ]
 
 

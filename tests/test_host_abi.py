@@ -188,3 +188,13 @@ def test_convert_inference_checkpoint_roundtrip(pkg, tmp_path):
 
 def test_host_sigma_schedule_matches_oracle(pkg):
     torch.testing.assert_close(pkg.sigma_schedule(10), oracle.sigma_schedule(10), rtol=0, atol=0)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The whole grid runs on one GPU; bench.py says so instead of pretending to scale."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 2
+    assert "ONE GPU" in (r.stdout + r.stderr)

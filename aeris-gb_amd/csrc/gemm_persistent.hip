@@ -35,8 +35,16 @@ constexpr int SMEM = A_STAGES * A_BYTES + B_STAGES * B_BYTES;  // 160 KB: all of
 constexpr int GM = 4;                     // row panels per L2 group
 }  // namespace
 
-template <int ACT, bool OUT_F32>
-__global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams p) {
+// PLAIN: no gate and no residual (qkv, fc1): the epilogue is compiled without those paths - about 2 % faster than
+// deciding at run time, block by block, that there is nothing to load
+template <int ACT, bool OUT_F32, bool PLAIN>
+__global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams p_in) {
+  GemmParams p = p_in;
+  if (PLAIN) {
+    p.gate = nullptr;
+    p.residual = nullptr;
+    p.res_dtype = -1;
+  }
   constexpr bool SWIGLU = ACT == AERIS_ACT_SWIGLU;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
@@ -517,13 +525,15 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 
 hipError_t gemm_persistent_configure() {
   hipError_t e;
-#define CFG(A, F32)                                                                                        \
-  e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_persistent_kernel<A, F32>),             \
+#define CFG1(A, F32, PL)                                                                                   \
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_persistent_kernel<A, F32, PL>),         \
                           hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);                                 \
   if (e != hipSuccess) return e;
+#define CFG(A, F32) CFG1(A, F32, false) CFG1(A, F32, true)
   CFG(AERIS_ACT_NONE, false) CFG(AERIS_ACT_NONE, true) CFG(AERIS_ACT_GELU, false) CFG(AERIS_ACT_GELU, true)
   CFG(AERIS_ACT_SWIGLU, false) CFG(AERIS_ACT_SWIGLU, true)
 #undef CFG
+#undef CFG1
   return hipSuccess;
 }
 
@@ -539,15 +549,22 @@ hipError_t gemm_persistent_launch(const GemmParams& p0, hipStream_t stream) {
   p.bpx = p.per_xcd < 32 ? p.per_xcd : 32;  // 32 CUs per XCD, one workgroup each
   dim3 grid(8 * p.bpx), block(NT);
   const bool f32 = p.c_dtype == AERIS_F32;
+  const bool plain = !p.gate && p.res_dtype < 0;
+#define GO1(A, F32)                                                                                        \
+  do {                                                                                                     \
+    if (plain) hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, F32, true>), grid, block, SMEM, stream, p);  \
+    else hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, F32, false>), grid, block, SMEM, stream, p);       \
+  } while (0)
 #define GO(A)                                                                                              \
   do {                                                                                                     \
-    if (f32) hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, true>), grid, block, SMEM, stream, p);    \
-    else hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, false>), grid, block, SMEM, stream, p);       \
+    if (f32) GO1(A, true);                                                                                   \
+    else GO1(A, false);                                                                                      \
   } while (0)
   if (swiglu) GO(AERIS_ACT_SWIGLU);
   else if (p.act == AERIS_ACT_GELU) GO(AERIS_ACT_GELU);
   else GO(AERIS_ACT_NONE);
 #undef GO
+#undef GO1
   return hipGetLastError();
 }
 

@@ -227,7 +227,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         if residual.numel() != M * N:
             raise RuntimeError("residual has the wrong size")
     big = gemm_uses_big_tiles(M, N, act) and act != "silu"
-    tag = f"gemm_256x256_{act or 'none'}_{'f32' if out.dtype == torch.float32 else 'bf16'}" if big else "gemm_128x128"
+    tag = "gemm_128x128"
+    if big:  # one tag per instantiation of the persistent kernel ("plain": neither gate nor residual in the epilogue)
+        tag = (f"gemm_256x256_{act or 'none'}_{'f32' if out.dtype == torch.float32 else 'bf16'}"
+               + ("_plain" if gate is None and residual is None else ""))
     with _timed(tag, 2.0 * M * n_w * K, "flop"):
         L.call("aeris_gemm_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), g_ptr, _ptr(residual), M, N, K,
                N, _ACT[act], _DT[residual.dtype] if residual is not None else 0, _DT[out.dtype], gstride,

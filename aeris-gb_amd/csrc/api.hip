@@ -112,35 +112,54 @@ int aeris_shift_region_ids(int H, int W, int ws_y, int ws_x, int shift_y, int sh
   return AERIS_OK;
 }
 
-int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
-                               int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
-                               void* stream) {
-  if (!qkv || !out) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: qkv/out is NULL");
-  if (!aligned16(qkv) || !aligned16(out)) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: qkv/out must be 16-byte aligned");
-  if (heads <= 0 || head_dim <= 0) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: heads/head_dim must be positive");
+static int window_attention_impl(const char* who, const void* qkv, void* out, const void* bias_table, int B, int H, int W,
+                                 int heads, int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask,
+                                 float scale, int64_t tok_stride, int64_t head_stride, int64_t part_stride, void* stream) {
+  if (!qkv || !out) return fail(AERIS_EINVAL, "%s: qkv/out is NULL", who);
+  if (!aligned16(qkv) || !aligned16(out)) return fail(AERIS_EINVAL, "%s: qkv/out must be 16-byte aligned", who);
+  if (heads <= 0 || head_dim <= 0) return fail(AERIS_EINVAL, "%s: heads/head_dim must be positive", who);
   if (int rc = check_window_geometry(B, H, W, ws_y, ws_x, shift_y, shift_x)) return rc;
-  if (!(scale > 0.f)) return fail(AERIS_EINVAL, "aeris_window_attention_fwd: scale must be positive");
+  if (!(scale > 0.f)) return fail(AERIS_EINVAL, "%s: scale must be positive", who);
   const bool small = aeris::attention_supported(ws_y, ws_x, head_dim);
   const bool masked = use_mask && (shift_y > 0 || shift_x > 0);
   if (!small && !aeris::attention_stream_supported(ws_y, ws_x, head_dim, bias_table != nullptr, masked))
     return fail(AERIS_EUNSUPPORTED,
-                "aeris_window_attention_fwd: no kernel for window %dx%d head_dim %d%s (built: 8x8, 12x12, 16x16 with head_dim "
+                "%s: no kernel for window %dx%d head_dim %d%s (built: 8x8, 12x12, 16x16 with head_dim "
                 "32 or 64, bias and mask optional; any window of up to 4096 tokens with head_dim 64 or 128 without bias and mask)",
-                ws_y, ws_x, head_dim, bias_table ? " with a bias table" : (masked ? " with the shift mask" : ""));
+                who, ws_y, ws_x, head_dim, bias_table ? " with a bias table" : (masked ? " with the shift mask" : ""));
   const int64_t units = (int64_t)B * (H / ws_y) * (W / ws_x) * heads;
   if (units > 0x7fffffffLL || (!small && (units + 8) * (((int64_t)ws_y * ws_x + 127) / 128) > 0x7fffffffLL))
-    return fail(AERIS_EUNSUPPORTED, "aeris_window_attention_fwd: more than 2^31-1 workgroups");
+    return fail(AERIS_EUNSUPPORTED, "%s: more than 2^31-1 workgroups", who);
   if (int rc = ensure_init()) return rc;
   if (!small) {
     hipError_t e = aeris::attention_stream_launch(qkv, out, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x, scale,
-                                                  reinterpret_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "aeris_window_attention_fwd launch (streaming kernel)");
+                                                  tok_stride, head_stride, part_stride, reinterpret_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "window attention launch (streaming kernel)");
     return AERIS_OK;
   }
   hipError_t e = aeris::attention_launch(qkv, out, bias_table, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x,
-                                         use_mask, scale, reinterpret_cast<hipStream_t>(stream));
-  if (e != hipSuccess) return hip_fail(e, "aeris_window_attention_fwd launch");
+                                         use_mask, scale, tok_stride, head_stride, part_stride,
+                                         reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "window attention launch");
   return AERIS_OK;
+}
+
+int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
+                               int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
+                               void* stream) {
+  const int64_t inner = (int64_t)heads * head_dim;
+  return window_attention_impl("aeris_window_attention_fwd", qkv, out, bias_table, B, H, W, heads, head_dim, ws_y, ws_x,
+                               shift_y, shift_x, use_mask, scale, 3 * inner, head_dim, inner, stream);
+}
+
+int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const void* bias_table, int B, int H, int W, int heads,
+                                     int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
+                                     int64_t plane_stride, void* stream) {
+  if (head_dim > 0 && B > 0 && H > 0 && W > 0 && (plane_stride < (int64_t)B * H * W * head_dim || plane_stride % 8))
+    return fail(AERIS_EINVAL, "aeris_window_attention_heads_fwd: plane_stride must be a multiple of 8 and at least B*H*W*head_dim");
+  return window_attention_impl("aeris_window_attention_heads_fwd", qkv_planes, out, bias_table, B, H, W, heads, head_dim, ws_y,
+                               ws_x, shift_y, shift_x, use_mask, scale, head_dim, plane_stride, (int64_t)heads * plane_stride,
+                               stream);
 }
 
 int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,
@@ -181,8 +200,26 @@ int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, cons
   if ((int64_t)((M + 127) / 128) * ((N + 63) / 64) > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_fwd: too many tiles");
   if (int rc = ensure_init()) return rc;
   hipError_t e = aeris::gemm_launch(A, W, C, bias, gate, residual, M, N, K, ldc, act, res_dtype, c_dtype,
-                                    gate_batch_stride, rows_per_batch, reinterpret_cast<hipStream_t>(stream));
+                                    gate_batch_stride, rows_per_batch, 0, 0, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_gemm_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_gemm_heads_fwd(const void* A, const void* W, void* C, const void* bias, int64_t M, int N, int K, int head_dim,
+                         int64_t plane_stride, void* stream) {
+  if (!A || !W || !C) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: A/W/C is NULL");
+  if (M <= 0 || N <= 0 || K <= 0) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: M, N, K must be positive");
+  if (!aligned16(A) || !aligned16(W) || !aligned16(C)) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: A/W/C must be 16-byte aligned");
+  if (K % 64) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_heads_fwd: K=%d must be a multiple of 64", K);
+  if (head_dim <= 0 || head_dim % 8) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: head_dim=%d must be a positive multiple of 8", head_dim);
+  if (N % head_dim) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: N=%d is not a multiple of head_dim=%d", N, head_dim);
+  if (plane_stride < M * head_dim || plane_stride % 8)
+    return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: plane_stride must be a multiple of 8 and at least M * head_dim");
+  if ((int64_t)((M + 127) / 128) * ((N + 63) / 64) > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_heads_fwd: too many tiles");
+  if (int rc = ensure_init()) return rc;
+  hipError_t e = aeris::gemm_launch(A, W, C, bias, nullptr, nullptr, M, N, K, N, AERIS_ACT_NONE, -1, AERIS_BF16, 0, M, head_dim,
+                                    plane_stride, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_gemm_heads_fwd launch");
   return AERIS_OK;
 }
 

@@ -186,7 +186,7 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_nt_kernel(GemmParams p)
           if (gate_row) x *= gate_row[nn];
           v[e] = x;
         }
-        const int64_t off = m * p.ldc + n;
+        const int64_t off = m * c_row_stride(p) + c_col_off(p, n);
         if (VEC) {
           if (p.res_dtype == AERIS_BF16) {
             const u32x2 r = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
@@ -252,8 +252,11 @@ hipError_t gemm_configure_all() {
 
 hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, const float* gate,
                        const void* residual, int64_t M, int N, int K, int64_t ldc, int act, int res_dtype,
-                       int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, hipStream_t stream) {
+                       int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, int split, int64_t plane_stride,
+                       hipStream_t stream) {
   GemmParams p;
+  p.split = split;
+  p.plane_stride = plane_stride;
   p.A = reinterpret_cast<const uint16_t*>(A);
   p.W = reinterpret_cast<const uint16_t*>(W);
   p.C = C;
@@ -273,12 +276,12 @@ hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, 
   const bool big = (M >= 256) && (N % bn_out == 0 || N >= 4 * bn_out) &&
                    ((M + 255) / 256) * ((N + bn_out - 1) / bn_out) >= 256;
   // vector epilogue (8 / 16 byte accesses to C and the residual) needs 4-element alignment of every row
-  const bool vec = ((ldc & 3) == 0) && ((N & 3) == 0);
+  const bool vec = (split || (ldc & 3) == 0) && ((N & 3) == 0);
   if (!vec) return swiglu ? launch_gemm<128, 128, 2, 2, true, false>(p, stream) : launch_gemm<128, 128, 2, 2, false, false>(p, stream);
   // (gate rows must allow 16-byte loads: the stride between batch rows is a multiple of 4 floats)
   const bool aligned = (reinterpret_cast<uintptr_t>(gate) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0;
   // the persistent kernel addresses W through one buffer descriptor (31-bit size) and loads 16 bytes per lane into LDS
-  const bool dma_ok = (int64_t)(swiglu ? 2 : 1) * N * K * 2 < (int64_t(1) << 31) && (K % 32) == 0 &&
+  const bool dma_ok = (int64_t)(swiglu ? 2 : 1) * N * K * 2 < (int64_t(1) << 31) && (K % 64) == 0 &&
                       ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15) == 0;
   if (big && dma_ok && act != AERIS_ACT_SILU && (gate_batch_stride & 3) == 0 && aligned) return gemm_persistent_launch(p, stream);
   return swiglu ? launch_gemm<128, 128, 2, 2, true, true>(p, stream) : launch_gemm<128, 128, 2, 2, false, true>(p, stream);

@@ -15,6 +15,10 @@ struct GemmParams {
   int N;  // logical output columns
   int K;
   int64_t ldc;
+  // output as column blocks ("head planes"): element (m, n) at (n / split) * plane_stride + m * split + n % split
+  // instead of m * ldc + n; split = 0: plain row-major C.  split % 8 == 0, no residual in this mode.
+  int split;
+  int64_t plane_stride;
   int64_t gate_batch_stride;
   int64_t rows_per_batch;
   int tiles_n;
@@ -27,6 +31,13 @@ struct GemmParams {
   int res_dtype;  // -1 none, AERIS_BF16, AERIS_F32
   int c_dtype;
 };
+
+// offset of the group of columns starting at n (a group never straddles a column block) within its row, and the
+// stride between rows, for either output layout
+__device__ __forceinline__ int64_t c_col_off(const GemmParams& p, int n) {
+  return p.split ? (int64_t)(n / p.split) * p.plane_stride + n % p.split : (int64_t)n;
+}
+__device__ __forceinline__ int64_t c_row_stride(const GemmParams& p) { return p.split ? (int64_t)p.split : p.ldc; }
 
 __device__ __forceinline__ uint32_t swz_off(int row, int chunk) {
   // byte offset of 16-byte chunk `chunk` (0..7) of tile row `row` in a [rows][64] bf16 tile

@@ -265,6 +265,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       else if (!full && p.res_dtype == AERIS_BF16) n_ld = n - 4;
       const bool upper = col_ok && !full;  // bf16: the wanted 4 columns are the upper half of what was loaded
       const int n_g = col_ok ? n : n_wave;
+      const int64_t c_rs = c_row_stride(p), c_co = c_col_off(p, col_ok ? n : n_wave);  // where this lane's chunk goes in C
       f32x4 gt0 = {1.f, 1.f, 1.f, 1.f}, gt1 = {1.f, 1.f, 1.f, 1.f};
       if (gate_tile) {
         gt0 = *reinterpret_cast<const f32x4*>(gate_tile + n_g);
@@ -355,7 +356,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         for (int it = 0; it < 4; ++it) {
           const int64_t m = m_base + i * 32 + rrow + 8 * it;
           if (col_ok && m < p.M) {
-            uint16_t* cp = reinterpret_cast<uint16_t*>(p.C) + m * p.ldc + n;
+            uint16_t* cp = reinterpret_cast<uint16_t*>(p.C) + m * c_rs + c_co;
             if (full) *reinterpret_cast<u32x4*>(cp) = out[it];
             else *reinterpret_cast<u32x2*>(cp) = u32x2{out[it].x, out[it].y};
           }
@@ -435,7 +436,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
           const int64_t m = m_base + i * 32 + rrow + 8 * it;
-          if (m < p.M && n < N) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + m * p.ldc + n) = out[it];
+          if (m < p.M && n < N) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + m * c_row_stride(p) + c_col_off(p, n)) = out[it];
         }
       }
     }

@@ -28,6 +28,9 @@ namespace aeris {
 struct AttnParams {
   const uint16_t* qkv;
   uint16_t* out;
+  // where q / k / v of (token, head) start, in elements: part * part_stride + head * head_stride + token * tok_stride
+  // ([S, 3 * inner] rows: inner, head_dim, 3 * inner; head planes [3 * heads][S][head_dim]: heads * plane, plane, head_dim)
+  int64_t tok_stride, head_stride, part_stride;
   const uint16_t* table;  // [(2WS_Y-1)(2WS_X-1), heads] bf16
   int B, H, W, heads;
   int nWy, nWx;
@@ -91,7 +94,7 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
   const int wy = wrem / p.nWx, wx = wrem - wy * p.nWx;
   const int H = p.H, W = p.W;
   const int inner = p.heads * HD;
-  const int64_t ld_qkv = 3 * (int64_t)inner;
+  const int64_t ld_qkv = p.tok_stride;
   const int64_t img_base = (int64_t)b * H * W;
   const int y0 = wy * WS_Y + p.sy, x0 = wx * WS_X + p.sx;
 
@@ -112,7 +115,7 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     int qpos = (wave + ps * NWAVES) * 32 + l31;
     if (qpos >= L) qpos = L - 1;
     q_tok[ps] = token_row(qpos);
-    const uint16_t* qp = p.qkv + q_tok[ps] * ld_qkv + head * HD + hi * 8;
+    const uint16_t* qp = p.qkv + head * p.head_stride + q_tok[ps] * ld_qkv + hi * 8;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[ps][s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
   }
@@ -121,8 +124,8 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
   // loop iteration): K chunks, V as 4 keys x 8 d per thread, the head's bias column
   constexpr int K_ITEMS = LPAD * CH, V_ITEMS = (LPAD / 4) * CH;
   constexpr int KIT = (K_ITEMS + NT - 1) / NT, VIT = (V_ITEMS + NT - 1) / NT, BIT = HAS_BIAS ? (TBL + NT - 1) / NT : 1;
-  const uint16_t* kbase = p.qkv + inner + head * HD;
-  const uint16_t* vbase = p.qkv + 2 * inner + head * HD;
+  const uint16_t* kbase = p.qkv + p.part_stride + head * p.head_stride;
+  const uint16_t* vbase = p.qkv + 2 * p.part_stride + head * p.head_stride;
   u32x4 kreg[KIT], vreg[VIT][4];
   float breg[BIT];
 #pragma unroll
@@ -325,17 +328,24 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
         }
       }
 
-    // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i]
-    if (q_valid) {
-      uint16_t* op = p.out + q_tok[ps] * inner + head * HD + hi * 4;
+    // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i].  The two lanes of a query (l31 and
+    // l31 + 32) each hold half of every 16-byte piece of the row; v_permlane32_swap on the pieces 2m and 2m + 1
+    // gives the lower lane all of piece 2m and the upper lane all of piece 2m + 1: half as many store
+    // instructions, and 32 contiguous bytes per row and instruction instead of 16.
+    {
+      uint16_t* op = p.out + q_tok[ps] * inner + head * HD + hi * 8;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2 w2;
-          w2.x = pack_bf16x2(o[db][g * 4] * inv, o[db][g * 4 + 1] * inv);
-          w2.y = pack_bf16x2(o[db][g * 4 + 2] * inv, o[db][g * 4 + 3] * inv);
-          *reinterpret_cast<u32x2*>(op + db * 32 + g * 8) = w2;
+        for (int m = 0; m < 2; ++m) {
+          const int g0 = 2 * m, g1 = 2 * m + 1;
+          const uint32_t x0 = pack_bf16x2(o[db][g0 * 4] * inv, o[db][g0 * 4 + 1] * inv);
+          const uint32_t x1 = pack_bf16x2(o[db][g0 * 4 + 2] * inv, o[db][g0 * 4 + 3] * inv);
+          const uint32_t y0 = pack_bf16x2(o[db][g1 * 4] * inv, o[db][g1 * 4 + 1] * inv);
+          const uint32_t y1 = pack_bf16x2(o[db][g1 * 4 + 2] * inv, o[db][g1 * 4 + 3] * inv);
+          const auto rx = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+          const auto ry = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+          if (q_valid) *reinterpret_cast<u32x4*>(op + db * 32 + m * 16) = u32x4{rx[0], ry[0], rx[1], ry[1]};
         }
     }
   }
@@ -376,8 +386,9 @@ static hipError_t launch_attn(const AttnParams& p, hipStream_t stream) {
 
 hipError_t attention_launch(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
                             int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
-                            hipStream_t stream) {
+                            int64_t tok_stride, int64_t head_stride, int64_t part_stride, hipStream_t stream) {
   AttnParams p;
+  p.tok_stride = tok_stride; p.head_stride = head_stride; p.part_stride = part_stride;
   p.qkv = reinterpret_cast<const uint16_t*>(qkv);
   p.out = reinterpret_cast<uint16_t*>(out);
   p.table = reinterpret_cast<const uint16_t*>(bias_table);

@@ -26,6 +26,7 @@ namespace {
 struct StreamParams {
   const uint16_t* qkv;
   uint16_t* out;
+  int64_t tok_stride, head_stride, part_stride;  // q / k / v addressing, as in the one-window kernel
   int B, H, W, heads;
   int nWy, nWx, ws_y, ws_x;
   int sy, sx;
@@ -86,7 +87,7 @@ window_attention_stream_kernel(StreamParams p) {
   const int H = p.H, W = p.W;
   const int L = p.ws_y * p.ws_x;
   const int inner = p.heads * HD;
-  const int64_t ld_qkv = 3 * (int64_t)inner;
+  const int64_t ld_qkv = p.tok_stride;
   const int64_t img_base = (int64_t)b * H * W;
   const int y0 = wy * p.ws_y + p.sy, x0 = wx * p.ws_x + p.sx;
 
@@ -106,13 +107,13 @@ window_attention_stream_kernel(StreamParams p) {
   const int64_t q_row = img_base + tok[qpos];
   bf16x8 qf[KS];
   {
-    const uint16_t* qp = p.qkv + q_row * ld_qkv + head * HD + hi * 8;
+    const uint16_t* qp = p.qkv + head * p.head_stride + q_row * ld_qkv + hi * 8;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
   }
 
-  const uint16_t* kbase = p.qkv + img_base * ld_qkv + inner + head * HD;
-  const uint16_t* vbase = p.qkv + img_base * ld_qkv + 2 * inner + head * HD;
+  const uint16_t* kbase = p.qkv + img_base * ld_qkv + p.part_stride + head * p.head_stride;
+  const uint16_t* vbase = p.qkv + img_base * ld_qkv + 2 * p.part_stride + head * p.head_stride;
   const int nch = (L + KC - 1) / KC;
 
   u32x4 kreg[KIT], vreg[4];
@@ -288,8 +289,10 @@ hipError_t attention_stream_configure_all() {
 }
 
 hipError_t attention_stream_launch(const void* qkv, void* out, int B, int H, int W, int heads, int head_dim, int ws_y,
-                                   int ws_x, int shift_y, int shift_x, float scale, hipStream_t stream) {
+                                   int ws_x, int shift_y, int shift_x, float scale, int64_t tok_stride, int64_t head_stride,
+                                   int64_t part_stride, hipStream_t stream) {
   StreamParams p;
+  p.tok_stride = tok_stride; p.head_stride = head_stride; p.part_stride = part_stride;
   p.qkv = reinterpret_cast<const uint16_t*>(qkv);
   p.out = reinterpret_cast<uint16_t*>(out);
   p.B = B; p.H = H; p.W = W; p.heads = heads;

@@ -192,11 +192,14 @@ class Attention(nn.Module):
     def core(self, y, shift=(0, 0), out=None):
         """y bf16 [b, n, d] -> attention output before ``wo`` (bf16 [b*n, inner])."""
         b, n, _ = y.shape
-        qkv = ops.gemm(y, self.to_qkv.weight, self.to_qkv.bias,
-                       out=ops.workspace("qkv", (b, n, self.to_qkv.weight.shape[0]), torch.bfloat16, y.device))
-        return ops.window_attention(qkv.view(b * n, -1), b, self.image_shape, self.heads, self.head_dim,
+        # q, k, v leave the GEMM as one [b*n, head_dim] plane per part and head (the "(c h d) -> c h d" split of
+        # model.py:300 done by the store addresses): a window's rows are then contiguous runs for the attention kernel
+        qkv = ops.gemm_heads(y, self.to_qkv.weight, self.to_qkv.bias, self.head_dim,
+                             out=ops.workspace("qkv", (3 * self.heads, b * n, self.head_dim), torch.bfloat16, y.device))
+        return ops.window_attention(qkv, b, self.image_shape, self.heads, self.head_dim,
                                     self.window_size, shift, self.relative_position_bias_table,
-                                    self.shift_mask and (shift[0] > 0 or shift[1] > 0), self.scale, out=out)
+                                    self.shift_mask and (shift[0] > 0 or shift[1] > 0), self.scale, out=out,
+                                    head_planes=True)
 
     def forward(self, x, shift=(0, 0)):
         b, n, d = x.shape

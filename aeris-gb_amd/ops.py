@@ -126,13 +126,19 @@ def shift_region_ids(H, W, ws_y, ws_x, shift_y, shift_x) -> np.ndarray:
 def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], heads: int, head_dim: int,
                      window_size: Tuple[int, int], shift: Tuple[int, int] = (0, 0),
                      bias_table: Optional[torch.Tensor] = None, use_mask: bool = False,
-                     scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """qkv bf16 [B*H*W, 3*heads*head_dim] (natural token order) -> bf16 [B*H*W, heads*head_dim]."""
+                     scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                     head_planes: bool = False) -> torch.Tensor:
+    """qkv bf16 [B*H*W, 3*heads*head_dim] (natural token order) -> bf16 [B*H*W, heads*head_dim].
+
+    ``head_planes``: qkv is [3*heads, B*H*W, head_dim] instead (plane c*heads + h = part c of head h), the layout
+    ``gemm_heads`` writes."""
     H, W = image_shape
     inner = heads * head_dim
     _dev(qkv, "qkv", torch.bfloat16)
     if qkv.numel() != B * H * W * 3 * inner:
         raise RuntimeError(f"qkv has {qkv.numel()} elements, expected {B}*{H}*{W}*3*{inner}")
+    if head_planes and tuple(qkv.shape) != (3 * heads, B * H * W, head_dim):
+        raise RuntimeError(f"qkv planes must be [{3 * heads}, {B * H * W}, {head_dim}], got {tuple(qkv.shape)}")
     if bias_table is not None:
         _dev(bias_table, "bias_table", torch.bfloat16)
         n = (2 * window_size[0] - 1) * (2 * window_size[1] - 1)
@@ -146,9 +152,14 @@ def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], he
             raise RuntimeError("out has the wrong size")
     Lw = window_size[0] * window_size[1]
     with _timed("window_attention", 4.0 * B * H * W * Lw * inner, "flop"):
-        L.call("aeris_window_attention_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads, head_dim,
-               window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
-               float(head_dim ** -0.5 if scale is None else scale), _stream())
+        if head_planes:
+            L.call("aeris_window_attention_heads_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads,
+                   head_dim, window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
+                   float(head_dim ** -0.5 if scale is None else scale), B * H * W * head_dim, _stream())
+        else:
+            L.call("aeris_window_attention_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads, head_dim,
+                   window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
+                   float(head_dim ** -0.5 if scale is None else scale), _stream())
     return out
 
 
@@ -235,6 +246,35 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         L.call("aeris_gemm_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), g_ptr, _ptr(residual), M, N, K,
                N, _ACT[act], _DT[residual.dtype] if residual is not None else 0, _DT[out.dtype], gstride,
                rows_per_batch if rows_per_batch > 0 else M, _stream())
+    return out
+
+
+def gemm_heads(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], head_dim: int,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a[M, K] @ w[N, K]^T + bias as N / head_dim planes: bf16 [N / head_dim, M, head_dim] (see aeris_gemm_heads_fwd)."""
+    _dev(a, "a", torch.bfloat16)
+    _dev(w, "w", torch.bfloat16)
+    K = a.shape[-1]
+    M = a.numel() // K
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise RuntimeError(f"w must be [N, {K}], got {tuple(w.shape)}")
+    if bias is not None:
+        _dev(bias, "bias", torch.bfloat16)
+        if bias.numel() != N:
+            raise RuntimeError(f"bias must have {N} elements")
+    if head_dim <= 0 or N % head_dim:
+        raise RuntimeError(f"N={N} is not a multiple of head_dim={head_dim}")
+    if out is None:
+        out = torch.empty(N // head_dim, M, head_dim, dtype=torch.bfloat16, device=a.device)
+    else:
+        _dev(out, "out", torch.bfloat16)
+        if tuple(out.shape) != (N // head_dim, M, head_dim):
+            raise RuntimeError("out has the wrong shape")
+    big = gemm_uses_big_tiles(M, N, None)
+    with _timed("gemm_256x256_none_bf16_plain" if big else "gemm_128x128", 2.0 * M * N * K, "flop"):
+        L.call("aeris_gemm_heads_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), M, N, K, head_dim,
+               M * head_dim, _stream())
     return out
 
 

@@ -168,6 +168,39 @@ def test_window_attention_streaming_parity(pkg, cuda, case):
     assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
 
 
+HEAD_PLANE_CASES = [
+    # B, H, W, heads, hd, ws_y, ws_x, shift, bias, mask -- one-window kernel (small and large grids) and streaming kernel
+    (1, 48, 64, 3, 64, 16, 16, 8, True, True),
+    (2, 16, 24, 2, 64, 8, 8, 4, True, True),
+    (1, 36, 48, 8, 32, 12, 12, 6, True, False),
+    (1, 160, 160, 24, 64, 16, 16, 8, True, True),   # the 256x256 GEMM tiles write the planes
+    (1, 120, 120, 2, 128, 60, 60, 30, False, False),
+    (2, 40, 60, 3, 64, 20, 20, 10, False, False),
+]
+
+
+@pytest.mark.parametrize("case", HEAD_PLANE_CASES, ids=lambda c: f"B{c[0]}_{c[1]}x{c[2]}_h{c[3]}x{c[4]}_ws{c[5]}")
+def test_head_plane_layout_is_bit_identical(pkg, cuda, case):
+    """The to_qkv GEMM writing one [tokens, head_dim] plane per part and head, and the attention kernels reading
+    them, do the same arithmetic as the [tokens, 3*inner] path: planes == columns, attention outputs equal bit for bit."""
+    B, H, W, heads, hd, wsy, wsx, sh, has_bias, use_mask = case
+    g = torch.Generator().manual_seed(11 * H + W)
+    inner, S, K = heads * hd, B * H * W, 128
+    x = bf(torch.randn(S, K, generator=g)).to(cuda)
+    w = bf(torch.randn(3 * inner, K, generator=g) / math.sqrt(K)).to(cuda)
+    bias = bf(0.3 * torch.randn(3 * inner, generator=g)).to(cuda)
+    table = bf(0.7 * torch.randn((2 * wsy - 1) * (2 * wsx - 1), heads, generator=g)).to(cuda) if has_bias else None
+    qkv = pkg.ops.gemm(x, w, bias)
+    planes = pkg.ops.gemm_heads(x, w, bias, hd)
+    torch.cuda.synchronize()
+    assert planes.shape == (3 * heads, S, hd)
+    assert torch.equal(planes.permute(1, 0, 2).reshape(S, 3 * inner), qkv)
+    o1 = pkg.ops.window_attention(qkv, B, (H, W), heads, hd, (wsy, wsx), (sh, sh), table, use_mask)
+    o2 = pkg.ops.window_attention(planes, B, (H, W), heads, hd, (wsy, wsx), (sh, sh), table, use_mask, head_planes=True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o1).all() and torch.equal(o1, o2)
+
+
 def test_window_attention_streaming_rejects_bias_and_mask(pkg, cuda):
     qkv = torch.zeros(60 * 60, 3 * 128, dtype=torch.bfloat16, device=cuda)
     table = torch.zeros(119 * 119, 1, dtype=torch.bfloat16, device=cuda)

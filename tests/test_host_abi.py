@@ -98,6 +98,19 @@ def test_argument_validation_needs_no_gpu(pkg):
     assert h(p16, p16, p16, None, None, None, 8, 8, 64, 4, 0, 0, 0, 0, 0, None) == L.EINVAL  # ldc < N
     assert h(p16, p16, p16, None, None, None, 0, 8, 64, 8, 0, 0, 0, 0, 0, None) == L.EINVAL  # M
     assert h(p16, p16, p16, None, None, None, 8, 8, 64, 8, 9, 0, 0, 0, 0, None) == L.EINVAL  # act
+    # head-plane variants: same checks, plus the plane geometry
+    fh = lib.aeris_window_attention_heads_fwd
+    assert fh(None, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 256 * 64, None) == L.EINVAL
+    assert fh(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 256 * 64 - 8, None) == L.EINVAL  # planes overlap
+    assert "plane_stride" in L.last_error()
+    assert fh(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 256 * 64 + 4, None) == L.EINVAL  # not 16-byte planes
+    assert fh(p16, p16, None, 1, 16, 16, 2, 96, 16, 16, 0, 0, 0, 0.1, 256 * 96, None) == L.EUNSUPPORTED  # head_dim 96
+    hh = lib.aeris_gemm_heads_fwd
+    assert hh(p16, p16, p16, None, 8, 128, 100, 64, 8 * 64, None) == L.EUNSUPPORTED  # K % 64
+    assert hh(p16, p16, p16, None, 8, 100, 64, 64, 8 * 64, None) == L.EINVAL  # N % head_dim
+    assert hh(p16, p16, p16, None, 8, 128, 64, 60, 8 * 60, None) == L.EINVAL  # head_dim % 8
+    assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64 - 8, None) == L.EINVAL  # planes overlap
+    assert hh(p16, None, p16, None, 8, 128, 64, 64, 8 * 64, None) == L.EINVAL  # W NULL
     # small ops
     assert lib.aeris_modulation_linear_fwd(p16, p16, None, p16, 1, 8, 12, 0, 0, None) == L.EUNSUPPORTED
     assert lib.aeris_timestep_embedding_fwd(p16, p16, 1, 7, 10000.0, None) == L.EINVAL

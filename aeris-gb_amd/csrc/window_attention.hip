@@ -66,6 +66,15 @@ __device__ __forceinline__ uint32_t k_off(int key, int chunk) {
   return (uint32_t)(key * 80 + chunk * 16);
 }
 
+// XOR pattern of the 16-byte chunks of V^T row d: the fragment reads (16 lanes = 16 consecutive rows, same chunk) are
+// conflict-free.  The transposing writes, whose lanes hold rows 8 apart, keep 4-way bank conflicts: also folding
+// bits 4-5 of d onto bits 1-2 removes them (LDS conflict cycles -85 % in the counters) but costs address registers
+// the kernel does not have - it spilled and ran 14 % slower.
+template <bool SWZ>
+__device__ __forceinline__ int v_swz(int d) {
+  return SWZ ? (d & 15) : 0;
+}
+
 template <int WS_Y, int WS_X, int HD, bool HAS_BIAS>
 __global__ void __launch_bounds__(attn_threads(WS_Y, WS_X)) __attribute__((amdgpu_waves_per_eu(2)))
 window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workgroups share a CU
@@ -177,8 +186,8 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
         hi2.x = (vreg[it][0][w] >> 16) | (vreg[it][1][w] & 0xffff0000u);
         hi2.y = (vreg[it][2][w] >> 16) | (vreg[it][3][w] & 0xffff0000u);
         const int d0 = c * 8 + 2 * w, d1 = d0 + 1;
-        *reinterpret_cast<u32x2*>(sV + d0 * VROW + (((pos >> 1) ^ (Cfg::V_SWZ ? (d0 & 15) : 0)) << 4) + (pos & 1) * 8) = lo;
-        *reinterpret_cast<u32x2*>(sV + d1 * VROW + (((pos >> 1) ^ (Cfg::V_SWZ ? (d1 & 15) : 0)) << 4) + (pos & 1) * 8) = hi2;
+        *reinterpret_cast<u32x2*>(sV + d0 * VROW + (((pos >> 1) ^ v_swz<Cfg::V_SWZ>(d0)) << 4) + (pos & 1) * 8) = lo;
+        *reinterpret_cast<u32x2*>(sV + d1 * VROW + (((pos >> 1) ^ v_swz<Cfg::V_SWZ>(d1)) << 4) + (pos & 1) * 8) = hi2;
       }
     }
   }
@@ -211,16 +220,25 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     if (!q_valid) qpos = L - 1;
 
     // ---- S^T = K Q^T
+    // The K fragments of key block kb + 1 are read while the MFMAs of block kb run (left to itself the compiler
+    // reads each fragment right before its MFMA and exposes the LDS latency every time).
     f32x16 acc[NQ];
+    bf16x8 kf[2][KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) kf[0][s] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(l31, s * 2 + hi));
 #pragma unroll
     for (int kb = 0; kb < NQ; ++kb) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[kb][e] = 0.f;
+      if (kb + 1 < NQ) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(kb * 32 + l31, s * 2 + hi));
-        acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ps][s], acc[kb], 0, 0, 0);
+        for (int s = 0; s < KS; ++s)
+          kf[(kb + 1) & 1][s] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>((kb + 1) * 32 + l31, s * 2 + hi));
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb & 1][s], qf[ps][s], acc[kb], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     // acc[kb][4g+i] = <k[key], q[query]>, key = 32kb + 8g + 4hi + i, query = qpos
 
@@ -249,15 +267,27 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     float mrow = -INFINITY;
     if (HAS_BIAS) {
       const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb)
+      // the 4 bias vectors of a key block are read two blocks ahead of their use
+      f32x4 bvb[3][4];
+      auto load_b = [&](int kb, f32x4 (&bq)[4]) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int key0 = kb * 32 + g * 8 + hi * 4;
-          const bool valid = (LPAD == L) || key0 < L;
-          const int kk = valid ? key0 : 0;
+          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
           const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
-          const f32x4 bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+          bq[g] = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+        }
+      };
+      load_b(0, bvb[0]);
+      if (NQ > 1) load_b(1, bvb[1]);
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb) {
+        if (kb + 2 < NQ) load_b(kb + 2, bvb[(kb + 2) % 3]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const bool valid = (LPAD == L) || (kb * 32 + g * 8 + hi * 4) < L;
+          const f32x4 bv = bvb[kb % 3][g];
           float t[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
@@ -268,6 +298,8 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
           mrow = fmaxf(fmaxf(mrow, t[0]), t[1]);
           mrow = fmaxf(fmaxf(mrow, t[2]), t[3]);
         }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     } else {
 #pragma unroll
       for (int kb = 0; kb < NQ; ++kb)
@@ -285,13 +317,18 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     }
     mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
 
-    // ---- P = exp2(t - max), row sum, pack to bf16 (B operand of PV)
+    // ---- P = exp2(t - max), row sum, pack to bf16 (the B operand of PV), and O^T = V^T P^T, 16 keys at a time.
+    // PV step (kb, t2): k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one
+    // V^T chunk per 32-row block of O^T.  While the MFMAs of a step run, the V^T fragments of the next step are read
+    // and its P is formed: the VALU work hides the MFMAs, and the LDS latency is a whole step away.
     float sum = 0.f;
-    uint32_t pk[NQ][8];
+    uint32_t pkb[2][4];
+    bf16x8 vfb[2][DB];
+    auto exp_step = [&](int step, uint32_t (&pk)[4]) {
+      const int kb = step >> 1, t2 = step & 1;
 #pragma unroll
-    for (int kb = 0; kb < NQ; ++kb)
-#pragma unroll
-      for (int h2 = 0; h2 < 8; ++h2) {
+      for (int h = 0; h < 4; ++h) {
+        const int h2 = 4 * t2 + h;
         float e0, e1;
         if (HAS_BIAS) {
           e0 = __builtin_amdgcn_exp2f(acc[kb][2 * h2] - mrow);
@@ -301,32 +338,40 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
           e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -mrow));
         }
         sum += e0 + e1;
-        pk[kb][h2] = pack_bf16x2(e0, e1);
+        pk[h] = pack_bf16x2(e0, e1);
       }
-    sum += __shfl_xor(sum, 32, 64);
-    const float inv = __builtin_amdgcn_rcpf(sum);
-
-    // ---- O^T = V^T P^T
+    };
+    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
+      const int chunk = step * 2 + hi;  // 16-byte chunk of the row: 8 keys of this lane half
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int d = db * 32 + l31;
+        f[db] = *reinterpret_cast<const bf16x8*>(sV + d * VROW + ((chunk ^ v_swz<Cfg::V_SWZ>(d)) << 4));
+      }
+    };
     f32x16 o[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+    load_v(0, vfb[0]);
+    exp_step(0, pkb[0]);
 #pragma unroll
-    for (int kb = 0; kb < NQ; ++kb)
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        // k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one V^T chunk
-        u32x4 pw = {pk[kb][4 * t2], pk[kb][4 * t2 + 1], pk[kb][4 * t2 + 2], pk[kb][4 * t2 + 3]};
-        const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-        const int chunk = (kb * 32 + t2 * 16) / 8 + hi;  // 16-byte chunk of the row: 8 keys of this lane half
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const int d = db * 32 + l31;
-          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(sV + d * VROW + ((chunk ^ (Cfg::V_SWZ ? (d & 15) : 0)) << 4));
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, o[db], 0, 0, 0);
-        }
+    for (int step = 0; step < 2 * NQ; ++step) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (step + 1 < 2 * NQ) {
+        load_v(step + 1, vfb[(step + 1) & 1]);
+        exp_step(step + 1, pkb[(step + 1) & 1]);
       }
+      const uint32_t* pk = pkb[step & 1];
+      u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
+      const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfb[step & 1][db], pf, o[db], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    sum += __shfl_xor(sum, 32, 64);
+    const float inv = __builtin_amdgcn_rcpf(sum);
 
     // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i].  The two lanes of a query (l31 and
     // l31 + 32) each hold half of every 16-byte piece of the row; v_permlane32_swap on the pieces 2m and 2m + 1

@@ -183,16 +183,28 @@ window_attention_stream_kernel(StreamParams p) {
     const unsigned char* sV = sK + Cfg::K_BYTES;
 
     // ---- S^T = K Q^T for the 64 keys of the chunk: acc[kb][4g+i] = <k[key], q>, key = 64j + 32kb + 8g + 4hi + i
+    // The K fragments are read PF MFMAs ahead of their use (left to itself the compiler reads each one right before
+    // its MFMA and exposes the LDS latency every time).
     f32x16 acc[2];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[kb][e] = 0.f;
+    {
+      constexpr int PF = 2, NS = 2 * KS;
+      bf16x8 kfr[PF + 1];
+      auto read_k = [&](int t) {
+        const int row = (t / KS) * 32 + l31, ch = (t % KS) * 2 + hi;
+        return *reinterpret_cast<const bf16x8*>(sK + (HD == 64 ? off128(row, ch) : off256(row, ch)));
+      };
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const int row = kb * 32 + l31, ch = s * 2 + hi;
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + (HD == 64 ? off128(row, ch) : off256(row, ch)));
-        acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], acc[kb], 0, 0, 0);
+      for (int t = 0; t < PF; ++t) kfr[t] = read_k(t);
+#pragma unroll
+      for (int t = 0; t < NS; ++t) {
+        if (t + PF < NS) kfr[(t + PF) % (PF + 1)] = read_k(t + PF);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[t / KS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[t % (PF + 1)], qf[t % KS], acc[t / KS], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     if (j * KC + KC > L) {  // last, partial chunk (uniform): keys past the window do not take part
@@ -204,6 +216,16 @@ window_attention_stream_kernel(StreamParams p) {
           if (key >= L) acc[kb][e] = -INFINITY;
         }
     }
+
+    // PV step (kb, t2): k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one V^T
+    // chunk per 32-row block of O^T.  The fragments of a step are read one step ahead of its MFMAs.
+    bf16x8 vfb[2][DB];
+    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
+      const int ch = step * 2 + hi;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) f[db] = *reinterpret_cast<const bf16x8*>(sV + off128(db * 32 + l31, ch));
+    };
+    load_v(0, vfb[0]);  // in flight during the softmax arithmetic below
 
     // ---- online softmax (exp2 domain): new row max, rescale what has been accumulated if any max moved
     float cm = acc[0][0];
@@ -223,32 +245,36 @@ window_attention_stream_kernel(StreamParams p) {
         for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
       m = m_new;
     }
-    uint32_t pk[2][8];
+
+    // ---- P = exp2(s - m) for 16 keys at a time and O^T += V^T P^T: while the MFMAs of a step run, the P of the next
+    // step is formed (the VALU work hides the MFMAs) and its V^T fragments are read
+    uint32_t pkb[2][4];
+    auto exp_step = [&](int step, uint32_t (&pk)[4]) {
+      const int kb = step >> 1, t2 = step & 1;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int h2 = 0; h2 < 8; ++h2) {
+      for (int h = 0; h < 4; ++h) {
+        const int h2 = 4 * t2 + h;
         const float e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -m));
         const float e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -m));
         l += e0 + e1;
-        pk[kb][h2] = pack_bf16x2(e0, e1);
+        pk[h] = pack_bf16x2(e0, e1);
       }
-
-    // ---- O^T += V^T P^T
+    };
+    exp_step(0, pkb[0]);
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        // k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one V^T chunk
-        const u32x4 pw = {pk[kb][4 * t2], pk[kb][4 * t2 + 1], pk[kb][4 * t2 + 2], pk[kb][4 * t2 + 3]};
-        const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-        const int ch = kb * 4 + t2 * 2 + hi;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(sV + off128(db * 32 + l31, ch));
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, o[db], 0, 0, 0);
-        }
+    for (int step = 0; step < 4; ++step) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (step + 1 < 4) {
+        load_v(step + 1, vfb[(step + 1) & 1]);
+        exp_step(step + 1, pkb[(step + 1) & 1]);
       }
+      const uint32_t* pk = pkb[step & 1];
+      const u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
+      const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfb[step & 1][db], pf, o[db], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
     if (j + 1 < nch) store_chunk((j + 1) & 1);
     __syncthreads();

@@ -120,6 +120,8 @@ static int window_attention_impl(const char* who, const void* qkv, void* out, co
   if (heads <= 0 || head_dim <= 0) return fail(AERIS_EINVAL, "%s: heads/head_dim must be positive", who);
   if (int rc = check_window_geometry(B, H, W, ws_y, ws_x, shift_y, shift_x)) return rc;
   if (!(scale > 0.f)) return fail(AERIS_EINVAL, "%s: scale must be positive", who);
+  if ((int64_t)B * H * W > 0x7fffffffLL || tok_stride > 0x7fffffffLL)
+    return fail(AERIS_EUNSUPPORTED, "%s: more than 2^31-1 tokens or elements per token row", who);
   const bool small = aeris::attention_supported(ws_y, ws_x, head_dim);
   const bool masked = use_mask && (shift_y > 0 || shift_x > 0);
   if (!small && !aeris::attention_stream_supported(ws_y, ws_x, head_dim, bias_table != nullptr, masked))

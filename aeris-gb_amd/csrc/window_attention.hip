@@ -103,28 +103,30 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
   const int wy = wrem / p.nWx, wx = wrem - wy * p.nWx;
   const int H = p.H, W = p.W;
   const int inner = p.heads * HD;
-  const int64_t ld_qkv = p.tok_stride;
-  const int64_t img_base = (int64_t)b * H * W;
+  // token rows and the stride between them fit 32 bits (checked by the caller): one 32 x 32 -> 64-bit multiply-add per
+  // address instead of a 64 x 64 multiply
+  const uint32_t ld_qkv = (uint32_t)p.tok_stride;
+  const uint32_t img_base = (uint32_t)b * (uint32_t)(H * W);
   const int y0 = wy * WS_Y + p.sy, x0 = wx * WS_X + p.sx;
 
-  auto token_row = [&](int pos) -> int64_t {
+  auto token_row = [&](int pos) -> uint32_t {
     int Y = y0 + pos / WS_X;
     int X = x0 + pos % WS_X;
     if (Y >= H) Y -= H;
     if (X >= W) X -= W;
-    return img_base + (int64_t)Y * W + X;
+    return img_base + (uint32_t)Y * (uint32_t)W + (uint32_t)X;
   };
 
   // ---- Q fragments of both query groups of this wave (B operand): lane = query, 8 consecutive d per k16 step.
   // Issued first: they are needed only after the K / V traffic below.
   bf16x8 qf[2][KS];
-  int64_t q_tok[2];
+  uint32_t q_tok[2];
 #pragma unroll
   for (int ps = 0; ps < 2; ++ps) {
     int qpos = (wave + ps * NWAVES) * 32 + l31;
     if (qpos >= L) qpos = L - 1;
     q_tok[ps] = token_row(qpos);
-    const uint16_t* qp = p.qkv + head * p.head_stride + q_tok[ps] * ld_qkv + hi * 8;
+    const uint16_t* qp = p.qkv + head * p.head_stride + (uint64_t)q_tok[ps] * ld_qkv + hi * 8;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[ps][s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
   }
@@ -142,7 +144,7 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     const int idx = tid + it * NT, key = idx / CH, c = idx % CH;
     kreg[it] = u32x4{0u, 0u, 0u, 0u};
     if ((K_ITEMS % NT == 0 || idx < K_ITEMS) && (LPAD == L || key < L))  // both compile-time true for full windows
-      kreg[it] = *reinterpret_cast<const u32x4*>(kbase + token_row(key) * ld_qkv + c * 8);
+      kreg[it] = *reinterpret_cast<const u32x4*>(kbase + (uint64_t)token_row(key) * ld_qkv + c * 8);
   }
 #pragma unroll
   for (int it = 0; it < VIT; ++it) {
@@ -151,7 +153,7 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     for (int j = 0; j < 4; ++j) {
       vreg[it][j] = u32x4{0u, 0u, 0u, 0u};
       if ((V_ITEMS % NT == 0 || idx < V_ITEMS) && (LPAD == L || kg * 4 < L))
-        vreg[it][j] = *reinterpret_cast<const u32x4*>(vbase + token_row(kg * 4 + j) * ld_qkv + c * 8);
+        vreg[it][j] = *reinterpret_cast<const u32x4*>(vbase + (uint64_t)token_row(kg * 4 + j) * ld_qkv + c * 8);
     }
   }
   if (HAS_BIAS) {
@@ -378,7 +380,7 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     // gives the lower lane all of piece 2m and the upper lane all of piece 2m + 1: half as many store
     // instructions, and 32 contiguous bytes per row and instruction instead of 16.
     {
-      uint16_t* op = p.out + q_tok[ps] * inner + head * HD + hi * 8;
+      uint16_t* op = p.out + (uint64_t)q_tok[ps] * (uint32_t)inner + head * HD + hi * 8;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll

@@ -87,7 +87,7 @@ window_attention_stream_kernel(StreamParams p) {
   const int H = p.H, W = p.W;
   const int L = p.ws_y * p.ws_x;
   const int inner = p.heads * HD;
-  const int64_t ld_qkv = p.tok_stride;
+  const uint32_t ld_qkv = (uint32_t)p.tok_stride;  // token rows and their stride fit 32 bits: one 32 x 32 -> 64-bit multiply-add per address
   const int64_t img_base = (int64_t)b * H * W;
   const int y0 = wy * p.ws_y + p.sy, x0 = wx * p.ws_x + p.sx;
 
@@ -107,13 +107,13 @@ window_attention_stream_kernel(StreamParams p) {
   const int64_t q_row = img_base + tok[qpos];
   bf16x8 qf[KS];
   {
-    const uint16_t* qp = p.qkv + head * p.head_stride + q_row * ld_qkv + hi * 8;
+    const uint16_t* qp = p.qkv + head * p.head_stride + (uint64_t)(uint32_t)q_row * ld_qkv + hi * 8;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
   }
 
-  const uint16_t* kbase = p.qkv + img_base * ld_qkv + p.part_stride + head * p.head_stride;
-  const uint16_t* vbase = p.qkv + img_base * ld_qkv + 2 * p.part_stride + head * p.head_stride;
+  const uint16_t* kbase = p.qkv + img_base * (int64_t)ld_qkv + p.part_stride + head * p.head_stride;
+  const uint16_t* vbase = p.qkv + img_base * (int64_t)ld_qkv + 2 * p.part_stride + head * p.head_stride;
   const int nch = (L + KC - 1) / KC;
 
   u32x4 kreg[KIT], vreg[4];
@@ -125,7 +125,7 @@ window_attention_stream_kernel(StreamParams p) {
       const int idx = tid + it * NT, key = idx / CH, c = idx % CH;
       int kp = key0 + key;
       if (kp > L - 1) kp = L - 1;  // rows past the window: any valid row, their scores are masked
-      kreg[it] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)tok[kp] * ld_qkv + c * 8);
+      kreg[it] = *reinterpret_cast<const u32x4*>(kbase + (uint64_t)(uint32_t)tok[kp] * ld_qkv + c * 8);
     }
     if (v_item) {
       const int kg = tid / CH, c = tid % CH;
@@ -133,7 +133,7 @@ window_attention_stream_kernel(StreamParams p) {
       for (int jj = 0; jj < 4; ++jj) {
         int kp = key0 + kg * 4 + jj;
         if (kp > L - 1) kp = L - 1;
-        vreg[jj] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)tok[kp] * ld_qkv + c * 8);
+        vreg[jj] = *reinterpret_cast<const u32x4*>(vbase + (uint64_t)(uint32_t)tok[kp] * ld_qkv + c * 8);
       }
     }
   };

@@ -209,6 +209,16 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     int tile_m, tile_n;
     decode(r_done, tile_m, tile_n);
     const int64_t m_base = (int64_t)tile_m * BM + grp * (BM / WM);
+    // Row addressing: the first row of this wave group in C / the residual is a wave-uniform 64-bit base, a lane adds
+    // its row r (0..127, relative) times the row stride as a 24-bit multiply (strides < 2^23, checked at launch)
+    // instead of a 64 x 64-bit multiply per access.  rows_left <= 0: a group entirely below the matrix.
+    const int64_t rows_left64 = p.M - m_base;
+    const int rows_left = rows_left64 < BM / WM ? (int)rows_left64 : BM / WM;
+    const int ld24 = (int)p.ldc, rs24 = (int)c_row_stride(p);
+    // (the row offsets do not depend on the tile; recomputing them per tile keeps them out of the registers of the
+    // main loop, where the compiler would otherwise park all of them)
+    int rrow_t = rrow;
+    asm volatile("" : "+v"(rrow_t));
     const int n_wave = tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
     u32x2 bq_next[FN][4];  // loaded ahead of the last block's stores, used after them
     // Staging area of this wave, 32 rows of 128 B: the A stage that the loader fills next is idle during the
@@ -265,23 +275,27 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       else if (!full && p.res_dtype == AERIS_BF16) n_ld = n - 4;
       const bool upper = col_ok && !full;  // bf16: the wanted 4 columns are the upper half of what was loaded
       const int n_g = col_ok ? n : n_wave;
-      const int64_t c_rs = c_row_stride(p), c_co = c_col_off(p, col_ok ? n : n_wave);  // where this lane's chunk goes in C
+      // where this lane's chunk of row 0 goes in C / comes from in the residual
+      unsigned char* const c_lane =
+          reinterpret_cast<unsigned char*>(p.C) + (m_base * c_row_stride(p) + c_col_off(p, col_ok ? n : n_wave)) * 2;
       f32x4 gt0 = {1.f, 1.f, 1.f, 1.f}, gt1 = {1.f, 1.f, 1.f, 1.f};
       if (gate_tile) {
         gt0 = *reinterpret_cast<const f32x4*>(gate_tile + n_g);
         gt1 = *reinterpret_cast<const f32x4*>(gate_tile + n_g + (full ? 4 : 0));
       }
+      const unsigned char* const res_lane = reinterpret_cast<const unsigned char*>(p.residual) +
+                                            (m_base * p.ldc + n_ld) * (p.res_dtype == AERIS_BF16 ? 2 : 4);
       u32x4 rq[4][2];
       auto load_res = [&](int i) {
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          int64_t m = m_base + i * 32 + rrow + 8 * it;
-          if (m > p.M - 1) m = p.M - 1;
-          const int64_t off = m * p.ldc + n_ld;
+          int r = i * 32 + rrow_t + 8 * it;
+          if (r > rows_left - 1) r = rows_left - 1;  // rows below the matrix read its last row (may be negative: M >= 1)
+          const int64_t off = (int64_t)__mul24(r, ld24);
           if (p.res_dtype == AERIS_BF16) {
-            rq[it][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
+            rq[it][0] = *reinterpret_cast<const u32x4*>(res_lane + off * 2);
           } else {
-            const float* rp = reinterpret_cast<const float*>(p.residual) + off;
+            const float* rp = reinterpret_cast<const float*>(res_lane + off * 4);
             rq[it][0] = *reinterpret_cast<const u32x4*>(rp);
             rq[it][1] = *reinterpret_cast<const u32x4*>(rp + (full ? 4 : 0));
           }
@@ -354,9 +368,9 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         }
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          const int64_t m = m_base + i * 32 + rrow + 8 * it;
-          if (col_ok && m < p.M) {
-            uint16_t* cp = reinterpret_cast<uint16_t*>(p.C) + m * c_rs + c_co;
+          const int r = i * 32 + rrow_t + 8 * it;
+          if (col_ok && r < rows_left) {
+            unsigned char* cp = c_lane + (int64_t)__mul24(r, rs24) * 2;
             if (full) *reinterpret_cast<u32x4*>(cp) = out[it];
             else *reinterpret_cast<u32x2*>(cp) = u32x2{out[it].x, out[it].y};
           }
@@ -379,16 +393,18 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         const int i = u / NJ;
         int n = unit_col(u);
         if (n >= N) n = N - 4;
+        const unsigned char* const res_lane = reinterpret_cast<const unsigned char*>(p.residual) +
+                                              (m_base * p.ldc + n) * (p.res_dtype == AERIS_BF16 ? 2 : 4);
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          int64_t m = m_base + i * 32 + rrow + 8 * it;
-          if (m > p.M - 1) m = p.M - 1;
-          const int64_t off = m * p.ldc + n;
+          int r = i * 32 + rrow_t + 8 * it;
+          if (r > rows_left - 1) r = rows_left - 1;
+          const int64_t off = (int64_t)__mul24(r, ld24);
           if (p.res_dtype == AERIS_BF16) {
-            const u32x2 r2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.residual) + off);
+            const u32x2 r2 = *reinterpret_cast<const u32x2*>(res_lane + off * 2);
             rq[it] = u32x4{r2.x, r2.y, 0u, 0u};
           } else {
-            rq[it] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.residual) + off);
+            rq[it] = *reinterpret_cast<const u32x4*>(res_lane + off * 4);
           }
         }
       };
@@ -433,10 +449,12 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           load_bias(r_done + 1, bq_next);
         }
         const int n = unit_col(u);
+        unsigned char* const c_lane =
+            reinterpret_cast<unsigned char*>(p.C) + (m_base * c_row_stride(p) + c_col_off(p, n < N ? n : 0)) * 4;
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          const int64_t m = m_base + i * 32 + rrow + 8 * it;
-          if (m < p.M && n < N) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + m * c_row_stride(p) + c_col_off(p, n)) = out[it];
+          const int r = i * 32 + rrow_t + 8 * it;
+          if (r < rows_left && n < N) *reinterpret_cast<f32x4*>(c_lane + (int64_t)__mul24(r, rs24) * 4) = out[it];
         }
       }
     }

@@ -19,7 +19,10 @@
 //                (lane ^ 32); exp2 with scale*log2(e) folded into one FMA
 //   O^T = V^T P^T  P^T taken straight from the S^T accumulator registers as the B operand; the
 //                k-slot permutation this implies is mirrored in the V^T fragment reads
-//   store        4 consecutive d per lane (8 B) to the folded token row
+//   store        8 consecutive d per lane (16 B, after a lane-half swap) to the folded token row
+// LDS reads are software-pipelined by hand (K fragments one key block ahead, bias vectors two, V^T fragments one 16-key
+// step ahead of their use); q / k / v are addressed through strides, so they may be the columns of one [tokens, 3*inner]
+// matrix or one [tokens, head_dim] plane per part and head.
 #include "common.h"
 #include "kernels.h"
 

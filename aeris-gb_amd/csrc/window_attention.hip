@@ -12,9 +12,10 @@
 //   V  [L][HD]   global -> registers (4 keys x 8 d per thread) -> 4x8 register transpose ->
 //                LDS as V^T [HD][LPAD], key groups permuted so that a PV fragment is one ds_read_b128
 //   bias table   column of this head -> LDS as fp32 4-vectors R4[s] = (R[s..s+3]), R reversed and
-//                pre-multiplied by log2(e): the biases of 4 consecutive keys are one ds_read_b128
+//                divided by the scale: the biases of 4 consecutive keys are one ds_read_b128
 //   Q            global -> registers (MFMA B operand), never in LDS
-//   S^T = K Q^T  v_mfma_f32_32x32x16_bf16, accumulators: lane = one query, 16*NW... keys
+//   S^T = K Q^T  v_mfma_f32_32x32x16_bf16, accumulators: lane = one query, 16 keys per 32-key block; they start at the
+//                bias (read from LDS straight into them), so the bias costs no add and the accumulators no zero-fill
 //   softmax      in registers; lane = query so the row max / sum need one cross-lane exchange
 //                (lane ^ 32); exp2 with scale*log2(e) folded into one FMA
 //   O^T = V^T P^T  P^T taken straight from the S^T accumulator registers as the B operand; the
@@ -159,11 +160,12 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
         vreg[it][j] = *reinterpret_cast<const u32x4*>(vbase + (uint64_t)token_row(kg * 4 + j) * ld_qkv + c * 8);
     }
   }
+  const float inv_scale = 1.0f / p.scale;
   if (HAS_BIAS) {
 #pragma unroll
     for (int it = 0; it < BIT; ++it) {
       const int j = tid + it * NT;
-      breg[it] = j < TBL ? bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E : 0.f;  // R[j]
+      breg[it] = j < TBL ? bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * inv_scale : 0.f;  // R[j]
     }
   }
   // every load above is in flight before the first LDS write below waits for one of them
@@ -224,31 +226,47 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     const bool q_valid = qpos < L;
     if (!q_valid) qpos = L - 1;
 
-    // ---- S^T = K Q^T
-    // The K fragments of key block kb + 1 are read while the MFMAs of block kb run (left to itself the compiler
-    // reads each fragment right before its MFMA and exposes the LDS latency every time).
+    // ---- S^T = K Q^T (+ bias / scale: the accumulators start at the relative-position bias, in the domain of the raw
+    // scores, so that logit * log2e = c * acc and the bias costs neither an add nor a zero-fill)
+    // The K fragments - and the bias vectors - of key block kb + 1 are read while the MFMAs of block kb run (left to
+    // itself the compiler reads each fragment right before its MFMA and exposes the LDS latency every time).
+    const int qiy = qpos / WS_X, qix = qpos % WS_X;
+    const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
     f32x16 acc[NQ];
     bf16x8 kf[2][KS];
+    auto init_acc = [&](int kb) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+        if (HAS_BIAS) {
+          const int key0 = kb * 32 + g * 8 + hi * 4;
+          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
+          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
+          bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[kb][g * 4 + i] = bv[i];
+      }
+    };
 #pragma unroll
     for (int s = 0; s < KS; ++s) kf[0][s] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(l31, s * 2 + hi));
+    init_acc(0);
 #pragma unroll
     for (int kb = 0; kb < NQ; ++kb) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[kb][e] = 0.f;
       if (kb + 1 < NQ) {
 #pragma unroll
         for (int s = 0; s < KS; ++s)
           kf[(kb + 1) & 1][s] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>((kb + 1) * 32 + l31, s * 2 + hi));
+        init_acc(kb + 1);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s = 0; s < KS; ++s) acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb & 1][s], qf[ps][s], acc[kb], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // acc[kb][4g+i] = <k[key], q[query]>, key = 32kb + 8g + 4hi + i, query = qpos
+    // acc[kb][4g+i] = <k[key], q[query]> + bias / scale, key = 32kb + 8g + 4hi + i, query = qpos
 
     // ---- cyclic-shift mask: only windows touching the wrapped border carry more than one region
-    const int qiy = qpos / WS_X, qix = qpos % WS_X;
     if (my || mx) {
       const float neg = -100.0f / p.scale;  // becomes -100 after the scale multiply below
       const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
@@ -267,59 +285,22 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
           }
     }
 
-    // ---- row max of the logits (exp2 domain).  With a bias the logits are formed here (one FMA each);
-    // without one the max of the raw scores is enough (scale > 0) and the FMA moves into the exp2 argument.
+    // ---- row max of the logits (exp2 domain): the max of the raw scores is enough (scale > 0), the scale moves into
+    // the exp2 argument
     float mrow = -INFINITY;
-    if (HAS_BIAS) {
-      const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
-      // the 4 bias vectors of a key block are read two blocks ahead of their use
-      f32x4 bvb[3][4];
-      auto load_b = [&](int kb, f32x4 (&bq)[4]) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int key0 = kb * 32 + g * 8 + hi * 4;
-          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
-          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
-          bq[g] = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+    for (int kb = 0; kb < NQ; ++kb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const bool valid = (LPAD == L) || (kb * 32 + g * 8 + hi * 4) < L;
+        if (!valid) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[kb][g * 4 + i] = -INFINITY;
         }
-      };
-      load_b(0, bvb[0]);
-      if (NQ > 1) load_b(1, bvb[1]);
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb) {
-        if (kb + 2 < NQ) load_b(kb + 2, bvb[(kb + 2) % 3]);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const bool valid = (LPAD == L) || (kb * 32 + g * 8 + hi * 4) < L;
-          const f32x4 bv = bvb[kb % 3][g];
-          float t[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            t[i] = fmaf(acc[kb][g * 4 + i], c, bv[i]);
-            if (!valid) t[i] = -INFINITY;
-            acc[kb][g * 4 + i] = t[i];
-          }
-          mrow = fmaxf(fmaxf(mrow, t[0]), t[1]);
-          mrow = fmaxf(fmaxf(mrow, t[2]), t[3]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4]), acc[kb][g * 4 + 1]);
+        mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4 + 2]), acc[kb][g * 4 + 3]);
       }
-    } else {
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const bool valid = (LPAD == L) || (kb * 32 + g * 8 + hi * 4) < L;
-          if (!valid) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[kb][g * 4 + i] = -INFINITY;
-          }
-          mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4]), acc[kb][g * 4 + 1]);
-          mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4 + 2]), acc[kb][g * 4 + 3]);
-        }
-      mrow *= c;
-    }
+    mrow *= c;
     mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
 
     // ---- P = exp2(t - max), row sum, pack to bf16 (the B operand of PV), and O^T = V^T P^T, 16 keys at a time.
@@ -334,14 +315,8 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const int h2 = 4 * t2 + h;
-        float e0, e1;
-        if (HAS_BIAS) {
-          e0 = __builtin_amdgcn_exp2f(acc[kb][2 * h2] - mrow);
-          e1 = __builtin_amdgcn_exp2f(acc[kb][2 * h2 + 1] - mrow);
-        } else {
-          e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -mrow));
-          e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -mrow));
-        }
+        const float e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -mrow));
+        const float e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -mrow));
         sum += e0 + e1;
         pk[h] = pack_bf16x2(e0, e1);
       }

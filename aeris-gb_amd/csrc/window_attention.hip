@@ -72,8 +72,9 @@ __device__ __forceinline__ uint32_t k_off(int key, int chunk) {
 
 // XOR pattern of the 16-byte chunks of V^T row d: the fragment reads (16 lanes = 16 consecutive rows, same chunk) are
 // conflict-free.  The transposing writes, whose lanes hold rows 8 apart, keep 4-way bank conflicts: also folding
-// bits 4-5 of d onto bits 1-2 removes them (LDS conflict cycles -85 % in the counters) but costs address registers
-// the kernel does not have - it spilled and ran 14 % slower.
+// bits 4-5 of d onto bits 1-2 removes them (LDS conflict cycles -85 % in the counters), but the read addresses then
+// no longer share a base: kept in registers they spill (14 % slower), recomputed per step the extra VALU work costs
+// 2-3 % - the kernel is bound by its VALU work, not by the LDS.
 template <bool SWZ>
 __device__ __forceinline__ int v_swz(int d) {
   return SWZ ? (d & 15) : 0;

@@ -25,6 +25,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
+// acc + lo + hi of a packed bf16 pair, in fp32 (v_dot2c_f32_bf16 with a pair of ones)
+__device__ __forceinline__ float dot2_ones(uint32_t packed, float acc) {
+  const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), ones, acc, false);
+}
 
 // 64-lane wavefront sum, the same value in every lane.  Data-parallel-primitive adds inside the 16-lane rows (quad
 // permutes, half mirror, mirror), two row broadcasts across the rows, total read from lane 63: six VALU operations

@@ -318,8 +318,8 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
         const int h2 = 4 * t2 + h;
         const float e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -mrow));
         const float e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -mrow));
-        sum += e0 + e1;
         pk[h] = pack_bf16x2(e0, e1);
+        sum = dot2_ones(pk[h], sum);  // the row sum of what PV multiplies: the rounded values, one instruction per pair
       }
     };
     auto load_v = [&](int step, bf16x8 (&f)[DB]) {

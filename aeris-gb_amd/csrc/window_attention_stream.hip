@@ -256,8 +256,8 @@ window_attention_stream_kernel(StreamParams p) {
         const int h2 = 4 * t2 + h;
         const float e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -m));
         const float e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -m));
-        l += e0 + e1;
         pk[h] = pack_bf16x2(e0, e1);
+        l = dot2_ones(pk[h], l);  // the row sum of what PV multiplies: the rounded values, one instruction per pair
       }
     };
     exp_step(0, pkb[0]);

@@ -42,6 +42,17 @@ constexpr int MAX_L = 4096;
 __device__ __forceinline__ uint32_t off128(int row, int chunk) {
   return (uint32_t)((row >> 1) * 256 + (((((row & 1) << 3) | chunk) ^ ((row >> 1) & 7)) << 4));
 }
+// V^T tile (rows = d, 128 bytes = 64 keys each): the chunk XOR also takes bits 4-6 of the row.  With the thread -> (key
+// group, d piece) map of the V staging below, both the transposing 8-byte writes (16 lanes = 8 pieces 8 rows apart x 2
+// key groups in the two halves of a chunk) and the fragment reads (16 lanes = 16 consecutive rows) are free of bank
+// conflicts (LDS counters: 3.9 cycles per instruction each); with off128() and consecutive threads on the pieces of
+// one key group the writes were 8-way conflicts, 31 cycles per instruction, and took most of the kernel's LDS time.
+// (head_dim 64, where half of the threads stage V and the writes are 4-way conflicts, is faster with the plain
+// layout and thread order: measured, -8 % with this one.)
+template <int HD>
+__device__ __forceinline__ uint32_t vt_off(int d, int chunk) {
+  return (uint32_t)((d >> 1) * 256 + ((((d & 1) << 3) | (chunk ^ ((d >> 1) & 7) ^ (HD == 128 ? (d >> 4) & 7 : 0))) << 4));
+}
 // the same for 256-byte rows (16 chunks)
 __device__ __forceinline__ uint32_t off256(int row, int chunk) { return (uint32_t)(row * 256 + ((chunk ^ (row & 15)) << 4)); }
 
@@ -118,6 +129,12 @@ window_attention_stream_kernel(StreamParams p) {
 
   u32x4 kreg[KIT], vreg[4];
   const bool v_item = (V_ITEMS >= NT) || tid < V_ITEMS;  // head_dim 64: half of the threads carry a V piece
+  // V piece of this thread: 4 keys (key group v_kg of the chunk) x 8 d (piece v_c).  Lane bits 0-2 (and 4 for head_dim
+  // 128) select the piece - the lanes of a key group still cover whole rows of V - bit 3 the key group within a pair
+  // that shares a 16-byte chunk of V^T: see vt_off().
+  const int v_b3 = (tid >> 3) & 1, v_b4 = (tid >> 4) & 1, v_b5 = (tid >> 5) & 1;
+  const int v_c = HD == 128 ? 8 * v_b4 + (tid & 7) : tid % CH;
+  const int v_kg = HD == 128 ? 4 * (tid >> 6) + 2 * v_b3 + v_b5 : tid / CH;
   auto load_chunk = [&](int j) {
     const int key0 = j * KC;
 #pragma unroll
@@ -128,7 +145,7 @@ window_attention_stream_kernel(StreamParams p) {
       kreg[it] = *reinterpret_cast<const u32x4*>(kbase + (uint64_t)(uint32_t)tok[kp] * ld_qkv + c * 8);
     }
     if (v_item) {
-      const int kg = tid / CH, c = tid % CH;
+      const int kg = v_kg, c = v_c;
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         int kp = key0 + kg * 4 + jj;
@@ -149,7 +166,7 @@ window_attention_stream_kernel(StreamParams p) {
     // stored in the order 0, 2, 1, 3: the 8 keys one lane needs for a k16 step of PV (4hi..4hi+3 and
     // 8+4hi..8+4hi+3, the accumulator layout of S^T) are then one aligned 16-byte chunk.
     if (v_item) {
-      const int kg = tid / CH, c = tid % CH;
+      const int kg = v_kg, c = v_c;
       const int pos = (kg & ~3) | (((kg & 1) << 1) | ((kg >> 1) & 1));
 #pragma unroll
       for (int w = 0; w < 4; ++w) {  // word w holds d = 8c + 2w (low half) and 8c + 2w + 1 (high half)
@@ -159,12 +176,18 @@ window_attention_stream_kernel(StreamParams p) {
         hi2.x = (vreg[0][w] >> 16) | (vreg[1][w] & 0xffff0000u);
         hi2.y = (vreg[2][w] >> 16) | (vreg[3][w] & 0xffff0000u);
         const int d0 = c * 8 + 2 * w, d1 = d0 + 1;
-        *reinterpret_cast<u32x2*>(sV + off128(d0, pos >> 1) + (pos & 1) * 8) = lo;
-        *reinterpret_cast<u32x2*>(sV + off128(d1, pos >> 1) + (pos & 1) * 8) = hi2;
+        *reinterpret_cast<u32x2*>(sV + vt_off<HD>(d0, pos >> 1) + (pos & 1) * 8) = lo;
+        *reinterpret_cast<u32x2*>(sV + vt_off<HD>(d1, pos >> 1) + (pos & 1) * 8) = hi2;
       }
     }
   };
 
+  // head_dim 128: vt_off(32 db + l31, 2 step + hi) = vt_row + 4096 db + vt_x[step ^ db]: the row part and the four possible chunk parts
+  // of this lane (five registers instead of one address per step and row block)
+  const uint32_t vt_row = (uint32_t)((l31 >> 1) * 256 + (l31 & 1) * 128);
+  uint32_t vt_x[4];
+#pragma unroll
+  for (int sx = 0; sx < 4; ++sx) vt_x[sx] = (uint32_t)(((2 * sx) ^ hi ^ ((l31 >> 1) & 7) ^ (l31 >> 4)) << 4);
   const float c = p.scale * LOG2E;
   float m = -INFINITY, l = 0.f;
   f32x16 o[DB];
@@ -220,10 +243,12 @@ window_attention_stream_kernel(StreamParams p) {
     // PV step (kb, t2): k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one V^T
     // chunk per 32-row block of O^T.  The fragments of a step are read one step ahead of its MFMAs.
     bf16x8 vfb[2][DB];
-    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
-      const int ch = step * 2 + hi;
+    auto load_v = [&](int step, bf16x8 (&f)[DB]) {  // f[db] = V^T rows 32 db + l31, chunk step * 2 + hi: vt_off(), taken apart
 #pragma unroll
-      for (int db = 0; db < DB; ++db) f[db] = *reinterpret_cast<const bf16x8*>(sV + off128(db * 32 + l31, ch));
+      for (int db = 0; db < DB; ++db) {
+        if (HD == 128) f[db] = *reinterpret_cast<const bf16x8*>(sV + vt_row + db * 4096 + vt_x[step ^ db]);
+        else f[db] = *reinterpret_cast<const bf16x8*>(sV + vt_off<HD>(db * 32 + l31, step * 2 + hi));
+      }
     };
     load_v(0, vfb[0]);  // in flight during the softmax arithmetic below
 

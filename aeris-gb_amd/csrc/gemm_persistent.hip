@@ -1,6 +1,9 @@
 // Persistent bf16 MFMA GEMM for gfx950, 256x256 output tiles, k-tiles of 64:  C[M,N] = epilogue(A[M,K] * W[N,K]^T)
 //
-// Same fragment layout and LDS swizzle as the plain tile kernel (gemm.hip), built around what bounds it on MI355X:
+// Same LDS swizzle as the plain tile kernel (gemm.hip), built around what bounds it on MI355X:
+//   - v_mfma_f32_16x16x32_bf16, not 32x32x16: same FLOP per cycle and the same LDS bytes per FLOP (a fragment is
+//     16 rows x 32 k instead of 32 rows x 16 k), but on operands that change from instruction to instruction the
+//     power-managed shader clock holds about 1.9 GHz with it against about 1.7 GHz with the larger shape
 //   - global loads go straight into LDS (buffer_load ... lds): no staging registers, no ds_write, and the lane ->
 //     address map of the load is the inverse of the LDS swizzle, so the tile lands in the layout the fragment reads
 //     want.  A load instruction fetches 8 rows x 128 B: whole cache lines (the CU's address unit takes 64-byte row
@@ -8,7 +11,7 @@
 //   - LDS holds two stages of the A tile and three of the W tile (160 KB); the loads of A run one k-tile ahead, those
 //     of W two, over the flat sequence (tile, k-tile), so the next tile's first k-tiles are in flight while the
 //     epilogue of the current tile runs (one workgroup per CU, persistent)
-//   - the two waves of a SIMD alternate memory slots (LDS fragment reads + load issue) and compute slots (16 MFMAs):
+//   - the two waves of a SIMD alternate memory slots (LDS fragment reads + load issue) and compute slots (32 MFMAs):
 //     a load instruction holds the issuing wave until the address unit has taken its 64 addresses, which would stall
 //     the MFMA stream if the computing wave issued it
 //   - tiles are ordered so that the workgroups resident on one XCD (blockIdx % 8) cover a contiguous chunk, 4 row
@@ -25,8 +28,8 @@ namespace aeris {
 namespace {
 constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 4;
 constexpr int NT = WM * WN * 64;          // 512 threads
-constexpr int FM = BM / WM / 32;          // 4
-constexpr int FN = BN / WN / 32;          // 2
+constexpr int FM = BM / WM / 16;          // 8 fragments of 16 rows
+constexpr int FN = BN / WN / 16;          // 4 fragments of 16 columns
 constexpr int A_BYTES = BM * BK * 2;      // 32 KB per stage of the A tile
 constexpr int B_BYTES = BN * BK * 2;      // 32 KB per stage of the W tile
 constexpr int A_STAGES = 2, B_STAGES = 3;
@@ -51,7 +54,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-  const int l31 = lane & 31, hi = lane >> 5;
+  const int l15 = lane & 15, q = lane >> 4;
   const int K = p.K, N = p.N;
   const int KT = K / BK;
 
@@ -150,51 +153,47 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     }
   };
 
-  // ---- fragment read offsets (per k16 step), relative to the stage of A / of W
-  uint32_t a_roff[4], b_roff[4];
+  // ---- fragment read offsets (per k-step of 32), relative to the stage of A / of W: lane (l15, q) reads the 8
+  // elements k = 32 ks + 8 q .. of row l15 of a 16-row fragment
+  uint32_t a_roff[2], b_roff[2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    a_roff[ks] = swz_off(wm * (BM / WM) + l31, ks * 2 + hi);
-    b_roff[ks] = swz_off(wn * (BN / WN) + l31, ks * 2 + hi);
+  for (int ks = 0; ks < 2; ++ks) {
+    a_roff[ks] = swz_off(wm * (BM / WM) + l15, ks * 4 + q);
+    b_roff[ks] = swz_off(wn * (BN / WN) + l15, ks * 4 + q);
   }
 
   // ---- accumulators.  They start a tile at the bias instead of zero: the bias add costs nothing that way.
-  // A lane's fragment columns are 4 consecutive n per (j, g): n = first column of the wave + 32 j + 8 g + 4 hi.
+  // A lane's fragment columns are 4 consecutive n per column fragment j: n = first column of the wave + 16 j + 4 q
+  // (SwiGLU: fragments 0, 1 are the gate columns, 2, 3 the up columns of the same 32 outputs).
   // N % 4 == 0, so a group of 4 is entirely inside or entirely outside the matrix (outside: clamped, computed,
   // never stored).
-  constexpr int NJ = SWIGLU ? 1 : FN;
-  f32x16 acc[FM][FN];
+  constexpr int NJ = SWIGLU ? FN / 2 : FN;  // column fragments of the output
+  f32x4 acc[FM][FN];
   auto wave_col0 = [&](int r) {  // first output column of this wave in tile r of the list
     int tile_m, tile_n;
     decode(r, tile_m, tile_n);
     return tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);
   };
-  auto load_bias = [&](int r, u32x2 (&bq)[FN][4]) {  // [SwiGLU: j = 0 gate bias, j = 1 up bias]
+  auto load_bias = [&](int r, u32x2 (&bq)[FN]) {
     const int n_wave = wave_col0(r);
 #pragma unroll
-    for (int j = 0; j < FN; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        int n = n_wave + (SWIGLU ? 0 : j * 32) + g * 8 + hi * 4;
-        if (n >= N) n = N - 4;
-        bq[j][g] = u32x2{0u, 0u};
-        if (p.bias) bq[j][g] = *reinterpret_cast<const u32x2*>(p.bias + (SWIGLU ? j * N : 0) + n);
-      }
+    for (int j = 0; j < FN; ++j) {
+      int n = n_wave + (SWIGLU ? (j & 1) : j) * 16 + q * 4;
+      if (n >= N) n = N - 4;
+      bq[j] = u32x2{0u, 0u};
+      if (p.bias) bq[j] = *reinterpret_cast<const u32x2*>(p.bias + (SWIGLU ? (j >> 1) * N : 0) + n);
+    }
   };
-  auto init_acc = [&](const u32x2 (&bq)[FN][4]) {
+  auto init_acc = [&](const u32x2 (&bq)[FN]) {
 #pragma unroll
-    for (int j = 0; j < FN; ++j)
+    for (int j = 0; j < FN; ++j) {
+      const f32x4 b = {bf16_lo(bq[j].x), bf16_hi(bq[j].x), bf16_lo(bq[j].y), bf16_hi(bq[j].y)};
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const float b[4] = {bf16_lo(bq[j][g].x), bf16_hi(bq[j][g].x), bf16_lo(bq[j][g].y), bf16_hi(bq[j][g].y)};
-#pragma unroll
-        for (int i = 0; i < FM; ++i)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] = b[e];
-      }
+      for (int i = 0; i < FM; ++i) acc[i][j] = b;
+    }
   };
   {
-    u32x2 bq[FN][4];
+    u32x2 bq[FN];
     load_bias(0, bq);
     init_acc(bq);
   }
@@ -220,7 +219,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     int rrow_t = rrow;
     asm volatile("" : "+v"(rrow_t));
     const int n_wave = tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
-    u32x2 bq_next[FN][4];  // loaded ahead of the last block's stores, used after them
+    u32x2 bq_next[FN];  // loaded ahead of the last block's stores, used after them
     // Staging area of this wave, 32 rows of 128 B: the A stage that the loader fills next is idle during the
     // epilogue, and the 4 KB of it that this wave's own loads will fill are written by nobody else.
     unsigned char* stg = smem + la_stage * A_BYTES + wave_u * 4096;
@@ -240,19 +239,16 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         else gate_per_lane = true;
       }
     }
-    // stage 1: activation on the 32 x 32 fragments of row block i, column block j (the bias is in the
+    // stage 1: activation on the 16 x 16 fragment of row fragment i, output column fragment j (the bias is in the
     // accumulators already).  The gate is applied after the staging, where a lane holds consecutive columns of
     // one row and needs far fewer gate registers.
-    auto fragment = [&](int i, int j, float (&v)[4][4]) {
+    auto fragment = [&](int i, int j, float (&v)[4]) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float x = acc[i][j][g * 4 + e];
-          if (SWIGLU) x = silu_f(x) * acc[i][1][g * 4 + e];
-          else if (ACT == AERIS_ACT_GELU) x = OUT_F32 ? gelu_erf_f(x) : gelu_bf16_f(x);
-          v[g][e] = x;
-        }
+      for (int e = 0; e < 4; ++e) {
+        float x = acc[i][j][e];
+        if (SWIGLU) x = silu_f(x) * acc[i][j + 2][e];
+        else if (ACT == AERIS_ACT_GELU) x = OUT_F32 ? gelu_erf_f(x) : gelu_bf16_f(x);
+        v[e] = x;
       }
     };
     auto gate_row_of = [&](int64_t m) {  // slow path: the tile straddles a batch boundary
@@ -303,24 +299,27 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       };
       if (p.res_dtype >= 0) load_res(0);
 #pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        // A row's 16-byte chunk c (8 columns) is split between lane l31 (columns 0-3) and lane l31 + 32 (4-7).
-        // v_permlane32_swap on the registers of chunks 2m and 2m+1 gives the lower lane all of chunk 2m and the
-        // upper lane all of chunk 2m+1: one conflict-free ds_write_b128 per lane and chunk pair instead of two
-        // 4-way conflicting ds_write_b64.
-        u32x2 w2[NJ * 4];
+      for (int i = 0; i < FM / 2; ++i) {  // blocks of 32 rows = two row fragments
+        // A row's 16-byte chunk (8 columns) of column fragment j is split between the lanes q = 0 / 1 (columns 0-3 /
+        // 4-7 of the fragment) or q = 2 / 3 (8-11 / 12-15).  v_permlane16_swap on the registers of fragments 2m and
+        // 2m+1 gives the lanes q = 0, 2 the two whole chunks of fragment 2m and the lanes q = 1, 3 those of fragment
+        // 2m+1: one ds_write_b128 per lane and fragment pair instead of two conflicting ds_write_b64.
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-          float v[4][4];
-          fragment(i, j, v);
+        for (int ii = 0; ii < 2; ++ii) {
+          u32x2 w2[NJ];
 #pragma unroll
-          for (int g = 0; g < 4; ++g) w2[j * 4 + g] = u32x2{pack_bf16x2(v[g][0], v[g][1]), pack_bf16x2(v[g][2], v[g][3])};
-        }
+          for (int j = 0; j < NJ; ++j) {
+            float v[4];
+            fragment(2 * i + ii, j, v);
+            w2[j] = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          }
 #pragma unroll
-        for (int mm = 0; mm < NJ * 2; ++mm) {
-          const auto rx = __builtin_amdgcn_permlane32_swap(w2[2 * mm].x, w2[2 * mm + 1].x, false, false);
-          const auto ry = __builtin_amdgcn_permlane32_swap(w2[2 * mm].y, w2[2 * mm + 1].y, false, false);
-          *reinterpret_cast<u32x4*>(stg + swz_off(l31, 2 * mm + hi)) = u32x4{rx[0], ry[0], rx[1], ry[1]};
+          for (int mm = 0; mm < NJ / 2; ++mm) {
+            const auto rx = __builtin_amdgcn_permlane16_swap(w2[2 * mm].x, w2[2 * mm + 1].x, false, false);
+            const auto ry = __builtin_amdgcn_permlane16_swap(w2[2 * mm].y, w2[2 * mm + 1].y, false, false);
+            *reinterpret_cast<u32x4*>(stg + swz_off(ii * 16 + l15, 4 * mm + 2 * (q & 1) + (q >> 1))) =
+                u32x4{rx[0], ry[0], rx[1], ry[1]};
+          }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -361,7 +360,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (i + 1 < FM) {
+        if (i + 1 < FM / 2) {
           if (p.res_dtype >= 0) load_res(i + 1);  // ahead of the stores below
         } else if (r_done + 1 < n_my) {
           load_bias(r_done + 1, bq_next);
@@ -377,20 +376,22 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         }
       }
     } else {
-      // stage 2 (f32 C): one 32 x 32 block per fragment, rows of 128 B (32 floats), 4 floats per lane and row
-      constexpr int UNITS = FM * NJ;
+      // stage 2 (f32 C): units of 32 rows x 32 columns (2 x 2 fragments), rows of 128 B (32 floats), 4 floats per
+      // lane and row
+      constexpr int NU = NJ / 2;  // units per block of 32 rows
+      constexpr int UNITS = FM / 2 * NU;
       u32x4 rq[4];
-      auto unit_col = [&](int u) { return n_wave + (u % NJ) * 32 + rch * 4; };
-      f32x4 gt[NJ];
+      auto unit_col = [&](int u) { return n_wave + (u % NU) * 32 + rch * 4; };
+      f32x4 gt[NU];
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
+      for (int j = 0; j < NU; ++j) {
         int n = unit_col(j);
         if (n >= N) n = N - 4;
         gt[j] = f32x4{1.f, 1.f, 1.f, 1.f};
         if (gate_tile) gt[j] = *reinterpret_cast<const f32x4*>(gate_tile + n);
       }
       auto load_res = [&](int u) {
-        const int i = u / NJ;
+        const int i = u / NU;
         int n = unit_col(u);
         if (n >= N) n = N - 4;
         const unsigned char* const res_lane = reinterpret_cast<const unsigned char*>(p.residual) +
@@ -411,14 +412,15 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       if (p.res_dtype >= 0) load_res(0);
 #pragma unroll
       for (int u = 0; u < UNITS; ++u) {
-        const int i = u / NJ, j = u % NJ;
-        float v[4][4];
-        fragment(i, j, v);
+        const int i = u / NU, j = u % NU;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          f32x4 w4 = {v[g][0], v[g][1], v[g][2], v[g][3]};
-          *reinterpret_cast<f32x4*>(stg + swz_off(l31, g * 2 + hi)) = w4;
-        }
+        for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            float v[4];
+            fragment(2 * i + ii, 2 * j + jj, v);
+            *reinterpret_cast<f32x4*>(stg + swz_off(ii * 16 + l15, jj * 4 + q)) = f32x4{v[0], v[1], v[2], v[3]};
+          }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -464,7 +466,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   // ---- flat pipeline over (tile, k-tile), ping-pong between the two wave groups.
   // Group 0 (wm = 0, one wave per SIMD) and group 1 (wm = 1, the other wave of each SIMD) run, per k-tile j, the
   // slots  M0 | C0 | M1 | C1 : a memory slot reads the fragments of half a k-tile (12 ds_read_b128) and issues 4
-  // loads, a compute slot issues the 16 MFMAs on those fragments.  Group 1 runs one slot behind group 0 and every
+  // loads, a compute slot issues the 32 MFMAs on those fragments.  Group 1 runs one slot behind group 0 and every
   // slot ends in a workgroup barrier: while one wave of a SIMD computes, the other one does its memory work.
   // Slots are numbered globally: group 0 runs k-tile j in slots 4j .. 4j+3, group 1 in 4j+1 .. 4j+4.
   //   A, two stages: the rows of A[j-1] that a group reads are last read in its M1(j-1); the group's own waves
@@ -503,14 +505,11 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         // ---- memory slot: LDS reads first (queued, non-blocking), then the loads
-        bf16x8 af[2][FM], bfr[2][FN];
+        bf16x8 af[FM], bfr[FN];
 #pragma unroll
-        for (int k2 = 0; k2 < 2; ++k2) {
+        for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(s_a + a_roff[half] + i * 16 * 128);
 #pragma unroll
-          for (int i = 0; i < FM; ++i) af[k2][i] = *reinterpret_cast<const bf16x8*>(s_a + a_roff[half * 2 + k2] + i * 32 * 128);
-#pragma unroll
-          for (int jn = 0; jn < FN; ++jn) bfr[k2][jn] = *reinterpret_cast<const bf16x8*>(s_w + b_roff[half * 2 + k2] + jn * 32 * 128);
-        }
+        for (int jn = 0; jn < FN; ++jn) bfr[jn] = *reinterpret_cast<const bf16x8*>(s_w + b_roff[half] + jn * 16 * 128);
         __builtin_amdgcn_sched_barrier(0);
         if (half == 0) issue_a();
         else issue_w();
@@ -522,12 +521,10 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_sched_barrier(0);
         // ---- compute slot
 #pragma unroll
-        for (int k2 = 0; k2 < 2; ++k2)
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-          for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int jn = 0; jn < FN; ++jn)
-              acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[k2][jn], af[k2][i], acc[i][jn], 0, 0, 0);
+          for (int jn = 0; jn < FN; ++jn)
+            acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[jn], af[i], acc[i][jn], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (half == 1) {
           if (more) __builtin_amdgcn_s_waitcnt(WAIT_VM4);
@@ -539,6 +536,10 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     }
     if (grp == 0) __builtin_amdgcn_s_barrier();
     epilogue(r);  // leaves the accumulators at the bias of the next tile
+    // Nothing that writes a register may be pending when the k-loop is entered: the compiler would guard the
+    // fragment registers with a wait for all vector memory operations inside the loop, on every k-tile, which
+    // cuts the lead of the W loads to one slot.  The first k-tile needs the oldest loads at once anyway.
+    __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   }
 }
 

@@ -281,8 +281,9 @@ hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, 
   // (gate rows must allow 16-byte loads: the stride between batch rows is a multiple of 4 floats)
   const bool aligned = (reinterpret_cast<uintptr_t>(gate) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0;
   // the persistent kernel addresses W through one buffer descriptor (31-bit size) and loads 16 bytes per lane into LDS
-  // ... and forms row offsets with 24-bit multiplies
+  // ... and forms row offsets with 24-bit multiplies, gate row offsets and batch numbers in 32 bits
   const bool dma_ok = (int64_t)(swiglu ? 2 : 1) * N * K * 2 < (int64_t(1) << 31) && (K % 64) == 0 && ldc < (1 << 23) && split < (1 << 23) &&
+                      gate_batch_stride < (int64_t(1) << 31) && (rows_per_batch <= 0 || M / rows_per_batch < (int64_t(1) << 31)) &&
                       ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15) == 0;
   if (big && dma_ok && act != AERIS_ACT_SILU && (gate_batch_stride & 3) == 0 && aligned) return gemm_persistent_launch(p, stream);
   return swiglu ? launch_gemm<128, 128, 2, 2, true, true>(p, stream) : launch_gemm<128, 128, 2, 2, false, true>(p, stream);

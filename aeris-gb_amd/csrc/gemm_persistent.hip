@@ -22,6 +22,7 @@
 #include "common.h"
 #include "gemm_common.h"
 #include "kernels.h"
+#include <type_traits>
 
 namespace aeris {
 
@@ -39,15 +40,19 @@ constexpr int GM = 4;                     // row panels per L2 group
 }  // namespace
 
 // PLAIN: no gate and no residual (qkv, fc1): the epilogue is compiled without those paths - about 2 % faster than
-// deciding at run time, block by block, that there is nothing to load
-template <int ACT, bool OUT_F32, bool PLAIN>
+// deciding at run time, block by block, that there is nothing to load.  RES_BF16: bf16 C with a bf16 residual (proj,
+// fc2 on a bf16 residual stream), compiled as a kernel of its own so that its deeper residual prefetch does not
+// share registers with the general path.
+template <int ACT, bool OUT_F32, bool PLAIN, bool RES_BF16 = false>
 __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams p_in) {
+  static_assert(!(PLAIN && RES_BF16) && !(OUT_F32 && RES_BF16), "RES_BF16 is a non-plain bf16-output form");
   GemmParams p = p_in;
   if (PLAIN) {
     p.gate = nullptr;
     p.residual = nullptr;
     p.res_dtype = -1;
   }
+  if (RES_BF16) p.res_dtype = AERIS_BF16;
   constexpr bool SWIGLU = ACT == AERIS_ACT_SWIGLU;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
@@ -203,8 +208,15 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   // before it.  The epilogue therefore loads everything it can ahead of its stores: the per-column operands
   // (gate) once per tile, the residual rows of the next 32-row block before the stores of the current one, the
   // bias of the next tile (for its accumulators) at the very start.
-  const int rrow = lane >> 3, rch = lane & 7;  // read-back mapping: row rrow + 8*it, 16-byte chunk rch
   auto epilogue = [&](int r_done) {
+    // Everything the epilogue derives from the lane number (staging addresses, column offsets, row offsets) does
+    // not depend on the tile; deriving it from a laundered copy of the lane number recomputes it per tile (a few
+    // dozen operations) and keeps it out of the registers of the main loop, where the compiler would otherwise
+    // park all of it.
+    int lane_t = lane;
+    asm volatile("" : "+v"(lane_t));
+    const int l15 = lane_t & 15, q = lane_t >> 4;
+    const int rrow = lane_t >> 3, rch = lane_t & 7;  // read-back mapping: row rrow + 8*it, 16-byte chunk rch
     int tile_m, tile_n;
     decode(r_done, tile_m, tile_n);
     const int64_t m_base = (int64_t)tile_m * BM + grp * (BM / WM);
@@ -214,10 +226,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     const int64_t rows_left64 = p.M - m_base;
     const int rows_left = rows_left64 < BM / WM ? (int)rows_left64 : BM / WM;
     const int ld24 = (int)p.ldc, rs24 = (int)c_row_stride(p);
-    // (the row offsets do not depend on the tile; recomputing them per tile keeps them out of the registers of the
-    // main loop, where the compiler would otherwise park all of them)
-    int rrow_t = rrow;
-    asm volatile("" : "+v"(rrow_t));
+    const int rrow_t = rrow;
     const int n_wave = tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
     u32x2 bq_next[FN];  // loaded ahead of the last block's stores, used after them
     // Staging area of this wave, 32 rows of 128 B: the A stage that the loader fills next is idle during the
@@ -226,8 +235,13 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 
     // gate: one row of p.gate per batch.  A tile whose rows are all in one batch (the usual case) loads its gate
     // columns once; otherwise every lane looks up the row of its own fragment row.
+    // The per-lane lookup avoids a 64-bit division per row: row r of the group (0..127) is in batch b0 if r < r1
+    // (r1 = first row of the next batch), else in batch b0 + 1 + (r - r1) / rows_per_batch, and that quotient of
+    // numbers below 128 is a multiply by ceil(2^16 / rows_per_batch) and a shift (0 when a batch has 128 rows or more).
     const float* gate_tile = nullptr;
     bool gate_per_lane = false;
+    int gate_b0 = 0, gate_r1 = 0;
+    uint32_t gate_magic = 0;
     if (p.gate) {
       if (p.gate_batch_stride == 0) {
         gate_tile = p.gate;
@@ -235,8 +249,14 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         int64_t last = m_base + BM / WM - 1;
         if (last > p.M - 1) last = p.M - 1;
         const int64_t b0 = m_base / p.rows_per_batch, b1 = last / p.rows_per_batch;
-        if (b0 == b1) gate_tile = p.gate + b0 * p.gate_batch_stride;
-        else gate_per_lane = true;
+        if (b0 == b1) {
+          gate_tile = p.gate + b0 * p.gate_batch_stride;
+        } else {
+          gate_per_lane = true;
+          gate_b0 = (int)b0;
+          gate_r1 = (int)((b0 + 1) * p.rows_per_batch - m_base);
+          if (p.rows_per_batch < BM / WM) gate_magic = (65536u + (uint32_t)p.rows_per_batch - 1u) / (uint32_t)p.rows_per_batch;
+        }
       }
     }
     // stage 1: activation on the 16 x 16 fragment of row fragment i, output column fragment j (the bias is in the
@@ -251,12 +271,99 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         v[e] = x;
       }
     };
-    auto gate_row_of = [&](int64_t m) {  // slow path: the tile straddles a batch boundary
-      if (m > p.M - 1) m = p.M - 1;
-      return p.gate + (m / p.rows_per_batch) * p.gate_batch_stride;
+    auto gate_row_of = [&](int r) {  // slow path: the group's rows straddle a batch boundary; r = row in the group
+      if (r > rows_left - 1) r = rows_left - 1;
+      const int d = r - gate_r1;
+      const int b = gate_b0 + (d < 0 ? 0 : 1 + (int)(((uint32_t)d * gate_magic) >> 16));
+      return p.gate + (int64_t)b * (int64_t)(int)p.gate_batch_stride;
     };
 
-    if (!OUT_F32) {
+    // bf16 C: block i of 32 rows (two row fragments) goes to the staging area as rows of 128 B, chunk-swizzled.
+    // A row's 16-byte chunk (8 columns) of column fragment j is split between the lanes q = 0 / 1 (columns 0-3 /
+    // 4-7 of the fragment) or q = 2 / 3 (8-11 / 12-15).  v_permlane16_swap on the registers of fragments 2m and
+    // 2m+1 gives the lanes q = 0, 2 the two whole chunks of fragment 2m and the lanes q = 1, 3 those of fragment
+    // 2m+1: one ds_write_b128 per lane and fragment pair instead of two conflicting ds_write_b64.
+    auto stage_block_bf16 = [&](int i) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+        u32x2 w2[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          float v[4];
+          fragment(2 * i + ii, j, v);
+          w2[j] = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        }
+#pragma unroll
+        for (int mm = 0; mm < NJ / 2; ++mm) {
+          const auto rx = __builtin_amdgcn_permlane16_swap(w2[2 * mm].x, w2[2 * mm + 1].x, false, false);
+          const auto ry = __builtin_amdgcn_permlane16_swap(w2[2 * mm].y, w2[2 * mm + 1].y, false, false);
+          *reinterpret_cast<u32x4*>(stg + swz_off(ii * 16 + l15, 4 * mm + 2 * (q & 1) + (q >> 1))) =
+              u32x4{rx[0], ry[0], rx[1], ry[1]};
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    // Interior tiles of the two forms that gain from it (bf16 residual with an optional per-tile gate: +5 % on
+    // K = 1536; plain GELU: +1 %; plain without activation measured 2 % slower this way and stays on the general
+    // path) take a path without any per-lane condition: every row and column of the group's 128 x 64 block is
+    // inside the matrix.  Straight-line code lets the compiler wait for exactly the loads a block needs (with the
+    // branches of the general path it waited for the next block's residual rows right after the stores), and the
+    // residual rows are requested two blocks ahead: block 0 at the start, block 1 once block 0's accumulators
+    // are staged and their registers free, blocks 2 and 3 after blocks 0 and 1 have been combined.
+    const bool interior = (RES_BF16 || (PLAIN && ACT == AERIS_ACT_GELU)) && !OUT_F32 && !SWIGLU &&
+                          rows_left == BM / WM && n_wave + BN / WN <= N && !gate_per_lane;
+    if (interior) {
+      const int n = n_wave + rch * 8;
+      unsigned char* const c_lane =
+          reinterpret_cast<unsigned char*>(p.C) + (m_base * c_row_stride(p) + c_col_off(p, n)) * 2;
+      f32x4 gt0 = {1.f, 1.f, 1.f, 1.f}, gt1 = {1.f, 1.f, 1.f, 1.f};
+      if (gate_tile) {
+        gt0 = *reinterpret_cast<const f32x4*>(gate_tile + n);
+        gt1 = *reinterpret_cast<const f32x4*>(gate_tile + n + 4);
+      }
+      const unsigned char* const res_lane =
+          reinterpret_cast<const unsigned char*>(p.residual) + (m_base * p.ldc + n) * 2;
+      u32x4 rq[FM / 2][4];
+      auto load_res = [&](int b) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+          rq[b][it] = *reinterpret_cast<const u32x4*>(res_lane + (int64_t)__mul24(b * 32 + rrow + 8 * it, ld24) * 2);
+      };
+      if (RES_BF16) load_res(0);
+#pragma unroll
+      for (int i = 0; i < FM / 2; ++i) {
+        stage_block_bf16(i);
+        if (RES_BF16 && i == 0) load_res(1);
+        u32x4 out[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + swz_off(rrow + 8 * it, rch));
+          if (RES_BF16) {
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { o[2 * e] = bf16_lo(w4[e]); o[2 * e + 1] = bf16_hi(w4[e]); }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { o[e] *= gt0[e]; o[4 + e] *= gt1[e]; }
+            const u32x4 r4 = rq[i][it];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { o[2 * e] += bf16_lo(r4[e]); o[2 * e + 1] += bf16_hi(r4[e]); }
+            w4 = u32x4{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
+          }
+          out[it] = w4;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        // the next loads go ahead of the stores below
+        if (RES_BF16 && i + 2 < FM / 2) load_res(i + 2);
+        if (i + 1 == FM / 2 && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+          *reinterpret_cast<u32x4*>(c_lane + (int64_t)__mul24(i * 32 + rrow + 8 * it, rs24) * 2) = out[it];
+      }
+    } else if (!OUT_F32) {
       // stage 2 (bf16 C): a whole 32 x 64 (SwiGLU: 32 x 32) block through LDS, rows of 128 B, chunk-swizzled; it
       // is read back as 16-byte chunks, 8 lanes per row, and C / residual are accessed as full row segments
       constexpr int CHUNKS = SWIGLU ? 4 : 8;  // 16-byte chunks (8 columns) per staged row
@@ -268,7 +375,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       // twice (f32)
       int n_ld = n;
       if (!col_ok) n_ld = n_wave;
-      else if (!full && p.res_dtype == AERIS_BF16) n_ld = n - 4;
+      else if (!full && (RES_BF16 || p.res_dtype == AERIS_BF16)) n_ld = n - 4;
       const bool upper = col_ok && !full;  // bf16: the wanted 4 columns are the upper half of what was loaded
       const int n_g = col_ok ? n : n_wave;
       // where this lane's chunk of row 0 goes in C / comes from in the residual
@@ -280,7 +387,8 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         gt1 = *reinterpret_cast<const f32x4*>(gate_tile + n_g + (full ? 4 : 0));
       }
       const unsigned char* const res_lane = reinterpret_cast<const unsigned char*>(p.residual) +
-                                            (m_base * p.ldc + n_ld) * (p.res_dtype == AERIS_BF16 ? 2 : 4);
+                                            (m_base * p.ldc + n_ld) * ((RES_BF16 || p.res_dtype == AERIS_BF16) ? 2 : 4);
+      const int res_dtype = RES_BF16 ? (int)AERIS_BF16 : p.res_dtype;
       u32x4 rq[4][2];
       auto load_res = [&](int i) {
 #pragma unroll
@@ -288,7 +396,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           int r = i * 32 + rrow_t + 8 * it;
           if (r > rows_left - 1) r = rows_left - 1;  // rows below the matrix read its last row (may be negative: M >= 1)
           const int64_t off = (int64_t)__mul24(r, ld24);
-          if (p.res_dtype == AERIS_BF16) {
+          if (res_dtype == AERIS_BF16) {
             rq[it][0] = *reinterpret_cast<const u32x4*>(res_lane + off * 2);
           } else {
             const float* rp = reinterpret_cast<const float*>(res_lane + off * 4);
@@ -297,44 +405,21 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           }
         }
       };
-      if (p.res_dtype >= 0) load_res(0);
+      if (res_dtype >= 0) load_res(0);
 #pragma unroll
       for (int i = 0; i < FM / 2; ++i) {  // blocks of 32 rows = two row fragments
-        // A row's 16-byte chunk (8 columns) of column fragment j is split between the lanes q = 0 / 1 (columns 0-3 /
-        // 4-7 of the fragment) or q = 2 / 3 (8-11 / 12-15).  v_permlane16_swap on the registers of fragments 2m and
-        // 2m+1 gives the lanes q = 0, 2 the two whole chunks of fragment 2m and the lanes q = 1, 3 those of fragment
-        // 2m+1: one ds_write_b128 per lane and fragment pair instead of two conflicting ds_write_b64.
-#pragma unroll
-        for (int ii = 0; ii < 2; ++ii) {
-          u32x2 w2[NJ];
-#pragma unroll
-          for (int j = 0; j < NJ; ++j) {
-            float v[4];
-            fragment(2 * i + ii, j, v);
-            w2[j] = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-          }
-#pragma unroll
-          for (int mm = 0; mm < NJ / 2; ++mm) {
-            const auto rx = __builtin_amdgcn_permlane16_swap(w2[2 * mm].x, w2[2 * mm + 1].x, false, false);
-            const auto ry = __builtin_amdgcn_permlane16_swap(w2[2 * mm].y, w2[2 * mm + 1].y, false, false);
-            *reinterpret_cast<u32x4*>(stg + swz_off(ii * 16 + l15, 4 * mm + 2 * (q & 1) + (q >> 1))) =
-                u32x4{rx[0], ry[0], rx[1], ry[1]};
-          }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        stage_block_bf16(i);
         u32x4 out[4];
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
           const int row = rrow + 8 * it;
           u32x4 w4 = *reinterpret_cast<const u32x4*>(stg + swz_off(row, rch));
-          if (p.gate || p.res_dtype >= 0) {
+          if (p.gate || res_dtype >= 0) {
             float o[8];
 #pragma unroll
             for (int e = 0; e < 4; ++e) { o[2 * e] = bf16_lo(w4[e]); o[2 * e + 1] = bf16_hi(w4[e]); }
             if (gate_per_lane) {
-              const float* gr = gate_row_of(m_base + i * 32 + row);
+              const float* gr = gate_row_of(i * 32 + row);
               gt0 = *reinterpret_cast<const f32x4*>(gr + n_g);
               gt1 = *reinterpret_cast<const f32x4*>(gr + n_g + (full ? 4 : 0));
             }
@@ -342,12 +427,12 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
 #pragma unroll
               for (int e = 0; e < 4; ++e) { o[e] *= gt0[e]; o[4 + e] *= gt1[e]; }
             }
-            if (p.res_dtype == AERIS_BF16) {
+            if (res_dtype == AERIS_BF16) {
               u32x4 r4 = rq[it][0];
               if (upper) { r4.x = r4.z; r4.y = r4.w; }
 #pragma unroll
               for (int e = 0; e < 4; ++e) { o[2 * e] += bf16_lo(r4[e]); o[2 * e + 1] += bf16_hi(r4[e]); }
-            } else if (p.res_dtype == AERIS_F32) {
+            } else if (res_dtype == AERIS_F32) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
                 o[e] += __uint_as_float(rq[it][0][e]);
@@ -361,7 +446,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (i + 1 < FM / 2) {
-          if (p.res_dtype >= 0) load_res(i + 1);  // ahead of the stores below
+          if (res_dtype >= 0) load_res(i + 1);  // ahead of the stores below
         } else if (r_done + 1 < n_my) {
           load_bias(r_done + 1, bq_next);
         }
@@ -432,7 +517,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           if (gate_per_lane) {
             int n = unit_col(u);
             if (n >= N) n = N - 4;
-            gt[j] = *reinterpret_cast<const f32x4*>(gate_row_of(m_base + i * 32 + row) + n);
+            gt[j] = *reinterpret_cast<const f32x4*>(gate_row_of(i * 32 + row) + n);
           }
           if (p.gate) o *= gt[j];
           if (p.res_dtype == AERIS_BF16) {
@@ -554,6 +639,12 @@ hipError_t gemm_persistent_configure() {
   CFG(AERIS_ACT_SWIGLU, false) CFG(AERIS_ACT_SWIGLU, true)
 #undef CFG
 #undef CFG1
+#define CFGR(A)                                                                                            \
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_persistent_kernel<A, false, false, true>), \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);                                 \
+  if (e != hipSuccess) return e;
+  CFGR(AERIS_ACT_NONE) CFGR(AERIS_ACT_GELU) CFGR(AERIS_ACT_SWIGLU)
+#undef CFGR
   return hipSuccess;
 }
 
@@ -570,6 +661,7 @@ hipError_t gemm_persistent_launch(const GemmParams& p0, hipStream_t stream) {
   dim3 grid(8 * p.bpx), block(NT);
   const bool f32 = p.c_dtype == AERIS_F32;
   const bool plain = !p.gate && p.res_dtype < 0;
+  const bool res_bf16 = !f32 && p.res_dtype == AERIS_BF16;
 #define GO1(A, F32)                                                                                        \
   do {                                                                                                     \
     if (plain) hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, F32, true>), grid, block, SMEM, stream, p);  \
@@ -577,7 +669,9 @@ hipError_t gemm_persistent_launch(const GemmParams& p0, hipStream_t stream) {
   } while (0)
 #define GO(A)                                                                                              \
   do {                                                                                                     \
-    if (f32) GO1(A, true);                                                                                   \
+    if (res_bf16)                                                                                            \
+      hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, false, false, true>), grid, block, SMEM, stream, p);  \
+    else if (f32) GO1(A, true);                                                                              \
     else GO1(A, false);                                                                                      \
   } while (0)
   if (swiglu) GO(AERIS_ACT_SWIGLU);

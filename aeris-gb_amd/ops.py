@@ -239,9 +239,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
             raise RuntimeError("residual has the wrong size")
     big = gemm_uses_big_tiles(M, N, act) and act != "silu"
     tag = "gemm_128x128"
-    if big:  # one tag per instantiation of the persistent kernel ("plain": neither gate nor residual in the epilogue)
+    if big:  # one tag per instantiation of the persistent kernel ("plain": neither gate nor residual in the epilogue;
+        # "res": bf16 output with a bf16 residual)
+        res_bf16 = residual is not None and residual.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
         tag = (f"gemm_256x256_{act or 'none'}_{'f32' if out.dtype == torch.float32 else 'bf16'}"
-               + ("_plain" if gate is None and residual is None else ""))
+               + ("_plain" if gate is None and residual is None else "_res" if res_bf16 else ""))
     with _timed(tag, 2.0 * M * n_w * K, "flop"):
         L.call("aeris_gemm_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), g_ptr, _ptr(residual), M, N, K,
                N, _ACT[act], _DT[residual.dtype] if residual is not None else 0, _DT[out.dtype], gstride,

@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Bytes that crossed the L2 <-> fabric boundary per launch at the config3 workload (average over the launches of
 # one step), from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a 1 GiB copy kernel; the summary
 # with the commands is profiles/denoiser_step_config3_pmc_traffic.txt.  Not measurable from inside this script.
-PMC_TRAFFIC_BYTES = {"config3": {"gemm_256x256_none_bf16": 34.786e9 + 3.185e9, "gemm_256x256_none_bf16_plain": 33.039e9 + 9.300e9,
+PMC_TRAFFIC_BYTES = {"config3": {"gemm_256x256_none_bf16_res": 34.786e9 + 3.185e9, "gemm_256x256_none_bf16_plain": 33.039e9 + 9.300e9,
                                  "gemm_256x256_gelu_bf16_plain": 30.902e9 + 12.740e9,
                                  "window_attention": 9.556e9 + 3.185e9, "norm_modulate": 3.186e9 + 3.185e9}}
 
@@ -245,12 +245,13 @@ def main():
         byts = 8.0 * S * wl["heads"] * wl["head_dim"]
         k["gbs"] = byts / (k["avg_ms"] * 1e-3) / 1e9
         k["frac_hbm_peak"] = k["gbs"] / PEAK_HBM_GBS
-    NAMES = {"gemm_256x256_none_bf16": "gemm_bf16_nt_persistent_kernel<0, false, false> (proj / fc2 GEMMs: x gate + residual)",
-             "gemm_256x256_none_bf16_plain": "gemm_bf16_nt_persistent_kernel<0, false, true> (qkv / embedding GEMMs)",
-             "gemm_256x256_gelu_bf16_plain": "gemm_bf16_nt_persistent_kernel<1, false, true> (fc1 GEMM + GELU)",
-             "gemm_256x256_none_f32": "gemm_bf16_nt_persistent_kernel<0, true, false>",
-             "gemm_256x256_none_f32_plain": "gemm_bf16_nt_persistent_kernel<0, true, true>",
-             "gemm_256x256_swiglu_bf16_plain": "gemm_bf16_nt_persistent_kernel<2, false, true>"}
+    NAMES = {"gemm_256x256_none_bf16_res": "gemm_bf16_nt_persistent_kernel<0, false, false, true> (proj / fc2 GEMMs: x gate + residual)",
+             "gemm_256x256_none_bf16": "gemm_bf16_nt_persistent_kernel<0, false, false, false>",
+             "gemm_256x256_none_bf16_plain": "gemm_bf16_nt_persistent_kernel<0, false, true, false> (qkv / embedding GEMMs)",
+             "gemm_256x256_gelu_bf16_plain": "gemm_bf16_nt_persistent_kernel<1, false, true, false> (fc1 GEMM + GELU)",
+             "gemm_256x256_none_f32": "gemm_bf16_nt_persistent_kernel<0, true, false, false>",
+             "gemm_256x256_none_f32_plain": "gemm_bf16_nt_persistent_kernel<0, true, true, false>",
+             "gemm_256x256_swiglu_bf16_plain": "gemm_bf16_nt_persistent_kernel<2, false, true, false>"}
     big = [t for t in kernels if t.startswith("gemm_256x256")]
     roofline = None
     if big:

@@ -45,6 +45,9 @@ GEMM_CASES = [
     # big tiles whose rows straddle a batch boundary (64 800 rows per batch = 253 tiles + 32 rows): per-lane gate rows
     (129600, 768, 256, None, True, 2, torch.bfloat16, torch.bfloat16),
     (129600, 512, 128, None, False, 2, torch.float32, torch.float32),
+    # 100 rows per batch: every 128-row group of a big tile straddles one or two batch boundaries
+    (64000, 512, 128, None, True, 640, torch.bfloat16, torch.bfloat16),
+    (64000, 256, 64, None, True, 640, torch.float32, torch.float32),
     (66000, 1028, 64, None, True, 0, torch.bfloat16, torch.bfloat16),  # big tiles, one k-tile, last 16-byte chunk half inside
     (70000, 1100, 128, "swiglu", True, 0, None, torch.bfloat16),  # big-tile SwiGLU with ragged N
     (300, 4096, 192, "gelu", True, 0, torch.bfloat16, torch.bfloat16),  # 2 x 16 big tiles: most workgroups idle or one tile

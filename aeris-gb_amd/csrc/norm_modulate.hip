@@ -1,5 +1,6 @@
 // Row norm (LayerNorm / RMSNorm) fused with the noise-level scale/shift modulation.  HBM-bound:
-// every row of x is read once and every row of y written once, 16 bytes per lane per access.
+// every row of x is read once and every row of y written once, 16 bytes per lane per access, both
+// marked non-temporal (streamed once: 4 % faster than with the default cache policy; either one alone is not).
 //
 // One wavefront owns one row at a time and keeps it in registers (NV vectors of 8 elements per
 // lane); the next row's loads are issued before the current row is reduced, so each wave has two
@@ -88,10 +89,11 @@ __global__ void __launch_bounds__(256) norm_modulate_kernel(NormParams p) {
       if (act[v]) {
         if (X_F32) {
           const float* xp = reinterpret_cast<const float*>(p.x) + row * d + col[v];
-          raw[v].a = *reinterpret_cast<const u32x4*>(xp);
-          raw[v].b = *reinterpret_cast<const u32x4*>(xp + 4);
+          raw[v].a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xp));
+          raw[v].b = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xp + 4));
         } else {
-          raw[v].a = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + row * d + col[v]);
+          raw[v].a = __builtin_nontemporal_load(
+              reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + row * d + col[v]));
         }
       }
     }
@@ -161,11 +163,11 @@ __global__ void __launch_bounds__(256) norm_modulate_kernel(NormParams p) {
       for (int e = 0; e < 8; ++e) o[e] = fmaf((u[v][e] - mean) * rstd, G[v][e], Bc[v][e]);
       if (p.y_dtype == AERIS_BF16) {
         u32x4 w = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
-        *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.y) + row * d + col[v]) = w;
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.y) + row * d + col[v]));
       } else {
         float* yp = reinterpret_cast<float*>(p.y) + row * d + col[v];
-        *reinterpret_cast<f32x4*>(yp) = f32x4{o[0], o[1], o[2], o[3]};
-        *reinterpret_cast<f32x4*>(yp + 4) = f32x4{o[4], o[5], o[6], o[7]};
+        __builtin_nontemporal_store(f32x4{o[0], o[1], o[2], o[3]}, reinterpret_cast<f32x4*>(yp));
+        __builtin_nontemporal_store(f32x4{o[4], o[5], o[6], o[7]}, reinterpret_cast<f32x4*>(yp + 4));
       }
     }
 #pragma unroll

@@ -315,7 +315,35 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     // are staged and their registers free, blocks 2 and 3 after blocks 0 and 1 have been combined.
     const bool interior = (RES_BF16 || (PLAIN && ACT == AERIS_ACT_GELU)) && !OUT_F32 && !SWIGLU &&
                           rows_left == BM / WM && n_wave + BN / WN <= N && !gate_per_lane;
-    if (interior) {
+    // Interior plain SwiGLU tiles skip the staging (in the read-back of the general path half of the lanes idle on
+    // its 64-byte rows; +2 %).  For the other forms this was slower (qkv -4 %, proj -5 %: 64-byte row pieces), although
+    // gate and residual are then applied in fp32 before the only rounding.
+    const bool interior_direct = SWIGLU && PLAIN && !OUT_F32 && rows_left == BM / WM && n_wave + 32 <= N;
+    if (interior_direct) {
+      // No staging: after a swap between lane rows (v_permlane16_swap on the registers of column fragments 2m and
+      // 2m + 1) lane (l15, q) owns 8 consecutive columns, 32 m + 16 (q & 1) + 8 (q >> 1) .., of row 16 i + l15: four
+      // lanes cover 64 contiguous bytes of a row of C, a store instruction 16 rows.
+      constexpr int NP = NJ / 2;
+      unsigned char* c_lane[NP];
+#pragma unroll
+      for (int m = 0; m < NP; ++m) {
+        const int n = n_wave + 32 * m + 16 * (q & 1) + 8 * (q >> 1);
+        c_lane[m] = reinterpret_cast<unsigned char*>(p.C) + (m_base * c_row_stride(p) + c_col_off(p, n)) * 2;
+      }
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        if (i + 1 == FM && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+#pragma unroll
+        for (int m = 0; m < NP; ++m) {
+          float a[4], b[4];
+          fragment(i, 2 * m, a);
+          fragment(i, 2 * m + 1, b);
+          const auto rx = __builtin_amdgcn_permlane16_swap(pack_bf16x2(a[0], a[1]), pack_bf16x2(b[0], b[1]), false, false);
+          const auto ry = __builtin_amdgcn_permlane16_swap(pack_bf16x2(a[2], a[3]), pack_bf16x2(b[2], b[3]), false, false);
+          *reinterpret_cast<u32x4*>(c_lane[m] + (int64_t)__mul24(i * 16 + l15, rs24) * 2) = u32x4{rx[0], ry[0], rx[1], ry[1]};
+        }
+      }
+    }     else if (interior) {
       const int n = n_wave + rch * 8;
       unsigned char* const c_lane =
           reinterpret_cast<unsigned char*>(p.C) + (m_base * c_row_stride(p) + c_col_off(p, n)) * 2;

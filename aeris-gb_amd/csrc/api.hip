@@ -176,6 +176,10 @@ int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, co
   if (kind != AERIS_NORM_LAYER && kind != AERIS_NORM_RMS) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: unknown norm kind %d", kind);
   if (order != AERIS_NORM_THEN_MOD && order != AERIS_MOD_THEN_NORM) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: unknown order %d", order);
   if (mod_batch_stride < 0) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: negative mod_batch_stride");
+  // the per-column parameters are read 16 bytes at a time
+  if (!aligned16(gamma) || (beta && !aligned16(beta)) || (shift && !aligned16(shift)) || (scale && !aligned16(scale)) ||
+      ((shift || scale) && (mod_batch_stride & 3)))
+    return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: gamma/beta/shift/scale must be 16-byte aligned, mod_batch_stride a multiple of 4");
   if (!(eps >= 0.f)) return fail(AERIS_EINVAL, "aeris_norm_modulate_fwd: eps must be non-negative");
   if (!aeris::norm_supported(d)) return fail(AERIS_EUNSUPPORTED, "aeris_norm_modulate_fwd: d=%d (need d %% 8 == 0 and d <= 6144)", d);
   hipError_t e = aeris::norm_modulate_launch(x, x_dtype, y, y_dtype, gamma, beta, param_dtype, shift, scale, mod_batch_stride, B,

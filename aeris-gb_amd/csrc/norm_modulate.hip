@@ -2,15 +2,16 @@
 // every row of x is read once and every row of y written once, 16 bytes per lane per access, both
 // marked non-temporal (streamed once: 4 % faster than with the default cache policy; either one alone is not).
 //
-// One wavefront owns one row at a time and keeps it in registers (NV vectors of 8 elements per
-// lane); the next row's loads are issued before the current row is reduced, so each wave has two
-// rows in flight.  Statistics are fp32: mean, then the centred second moment (LayerNorm), or the
-// plain second moment (RMSNorm).  The per-column parameters are folded once per wave into
+// One wavefront owns a row and keeps it in registers (NV vectors of 8 elements per lane).  Statistics are
+// fp32: mean, then the centred second moment (LayerNorm), or the plain second moment (RMSNorm).  The
+// per-column parameters are folded into
 //     pre :  u = x * P1 + P0          (P1 = 1 + scale, P0 = shift;  only for "modulate then norm")
 //     post:  y = n(u) * G + Bc        (G = gamma, Bc = beta, or for "norm then modulate"
 //                                      G = gamma*(1+scale), Bc = beta*(1+scale) + shift)
-// and stay in registers while the wave walks down its rows (re-folded when the batch index, and
-// with it the modulation row, changes).
+// Two kernels: rows of up to 2048 elements go to norm_modulate_block_kernel (no loop: a block of four
+// waves takes eight rows and folds the parameters once into LDS); longer rows to norm_modulate_kernel
+// (persistent waves walk down the rows with the folded parameters in registers, the next row's loads
+// issued before the current row is reduced).
 #include "common.h"
 #include "kernels.h"
 
@@ -175,10 +176,219 @@ __global__ void __launch_bounds__(256) norm_modulate_kernel(NormParams p) {
   }
 }
 
+// Rows of up to 2048 elements: a kernel without a loop.  A block of four waves takes 4 * ROWS consecutive rows of one
+// batch entry (wave w the rows w, w + 4, ...), requests all of them first, folds the per-column parameters once into
+// LDS while the rows are in flight (as fp32, the first and second four columns of a lane's eight in separate arrays so
+// that the 16-byte reads of neighbouring lanes do not share banks), and then normalises row by row.  Short-lived waves
+// with few registers (eight waves per SIMD) keep more bytes in flight and mix loads and stores more evenly than waves
+// that walk down the matrix: a plain copy reaches 5.85 TB/s this way against 5.3 TB/s with the persistent structure.
+template <int NV, bool X_F32, bool PRE, bool FULL, int ROWS>
+__global__ void __launch_bounds__(256) norm_modulate_block_kernel(NormParams p, int64_t blocks_per_batch) {
+  constexpr int GROUPS = NV * 64;  // column groups of 8 that the LDS arrays hold
+  __shared__ f32x4 sG[2][GROUPS], sB[2][GROUPS];
+  __shared__ f32x4 sP1[PRE ? 2 : 1][PRE ? GROUPS : 1], sP0[PRE ? 2 : 1][PRE ? GROUPS : 1];
+  typedef __attribute__((address_space(1))) const unsigned char* gc_ptr;
+  typedef __attribute__((address_space(1))) unsigned char* g_ptr;
+  const gc_ptr xg = (gc_ptr)p.x;
+  const g_ptr yg = (g_ptr)p.y;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int d = p.d;
+  const float inv_d = 1.0f / (float)d;
+  const int64_t b = (int64_t)blockIdx.x / blocks_per_batch;
+  const int64_t first = b * p.rows_per_batch + ((int64_t)blockIdx.x - b * blocks_per_batch) * (4 * ROWS);
+  int64_t end = (b + 1) * p.rows_per_batch;  // rows of this batch entry end here
+  if (end > p.rows) end = p.rows;
+
+  struct Raw { u32x4 a, b; };
+  Raw raw[ROWS][NV];
+#pragma unroll
+  for (int j = 0; j < ROWS; ++j) {
+    int64_t row = first + j * 4 + w;
+    if (row > end - 1) row = end - 1;  // past the end: the last row again, never stored
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int col = (v * 64 + lane) * 8;
+      raw[j][v].a = u32x4{0u, 0u, 0u, 0u};
+      raw[j][v].b = u32x4{0u, 0u, 0u, 0u};
+      if (FULL || col < d) {
+        if (X_F32) {
+          const gc_ptr xp = xg + (row * d + col) * 4;
+          raw[j][v].a = __builtin_nontemporal_load((const __attribute__((address_space(1))) u32x4*)xp);
+          raw[j][v].b = __builtin_nontemporal_load((const __attribute__((address_space(1))) u32x4*)(xp + 16));
+        } else {
+          raw[j][v].a = __builtin_nontemporal_load((const __attribute__((address_space(1))) u32x4*)(xg + (row * d + col) * 2));
+        }
+      }
+    }
+  }
+
+  // ---- fold the parameters of this batch entry: pre  u = x * P1 + P0,  post  y = n(u) * G + Bc.
+  // All loads of a column group are issued before the first of them is used (vector memory returns in order: a
+  // wait inside a chain of dependent loads would also wait for the rows requested above, once per link).  A
+  // pointer that is absent is replaced by one that is present and its values are discarded.
+  {
+    const float* sh = p.shift ? p.shift + (p.mod_batch_stride ? b * p.mod_batch_stride : 0) : nullptr;
+    const float* sc = p.scale ? p.scale + (p.mod_batch_stride ? b * p.mod_batch_stride : 0) : nullptr;
+    const bool has_mod = sh || sc, has_beta = p.beta != nullptr;
+    const float* shp = sh ? sh : sc;
+    const float* scp = sc ? sc : sh;
+    const void* betap = has_beta ? p.beta : p.gamma;
+    for (int g = threadIdx.x; g < GROUPS; g += 256) {
+      if (!(FULL || g * 8 < d)) continue;
+      f32x4 gv[2], bv[2], shv[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, scv[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+      u32x4 gq = {0u, 0u, 0u, 0u}, bq = {0u, 0u, 0u, 0u};
+      if (p.param_f32) {
+        gv[0] = reinterpret_cast<const f32x4*>(p.gamma)[2 * g];
+        gv[1] = reinterpret_cast<const f32x4*>(p.gamma)[2 * g + 1];
+        bv[0] = reinterpret_cast<const f32x4*>(betap)[2 * g];
+        bv[1] = reinterpret_cast<const f32x4*>(betap)[2 * g + 1];
+      } else {
+        gq = reinterpret_cast<const u32x4*>(p.gamma)[g];
+        bq = reinterpret_cast<const u32x4*>(betap)[g];
+      }
+      if (has_mod) {
+        shv[0] = reinterpret_cast<const f32x4*>(shp)[2 * g];
+        shv[1] = reinterpret_cast<const f32x4*>(shp)[2 * g + 1];
+        scv[0] = reinterpret_cast<const f32x4*>(scp)[2 * g];
+        scv[1] = reinterpret_cast<const f32x4*>(scp)[2 * g + 1];
+      }
+      float G[8], Bc[8], P1[8], P0[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float ga, be;
+        if (p.param_f32) {
+          ga = gv[e >> 2][e & 3];
+          be = bv[e >> 2][e & 3];
+        } else {
+          ga = (e & 1) ? bf16_hi(gq[e >> 1]) : bf16_lo(gq[e >> 1]);
+          be = (e & 1) ? bf16_hi(bq[e >> 1]) : bf16_lo(bq[e >> 1]);
+        }
+        if (!has_beta) be = 0.f;
+        const float s1 = sc ? 1.f + scv[e >> 2][e & 3] : 1.f;
+        const float s0 = sh ? shv[e >> 2][e & 3] : 0.f;
+        if (PRE) { P1[e] = s1; P0[e] = s0; G[e] = ga; Bc[e] = be; }
+        else { G[e] = ga * s1; Bc[e] = be * s1 + s0; }
+      }
+      sG[0][g] = f32x4{G[0], G[1], G[2], G[3]};  sG[1][g] = f32x4{G[4], G[5], G[6], G[7]};
+      sB[0][g] = f32x4{Bc[0], Bc[1], Bc[2], Bc[3]};  sB[1][g] = f32x4{Bc[4], Bc[5], Bc[6], Bc[7]};
+      if (PRE) {
+        sP1[0][g] = f32x4{P1[0], P1[1], P1[2], P1[3]};  sP1[1][g] = f32x4{P1[4], P1[5], P1[6], P1[7]};
+        sP0[0][g] = f32x4{P0[0], P0[1], P0[2], P0[3]};  sP0[1][g] = f32x4{P0[4], P0[5], P0[6], P0[7]};
+      }
+    }
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int j = 0; j < ROWS; ++j) {
+    const int64_t row = first + j * 4 + w;
+    float u[NV][8];
+    float s = 0.f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int g = v * 64 + lane;
+      const bool act = FULL || g * 8 < d;
+      if (X_F32) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          u[v][e] = __uint_as_float(raw[j][v].a[e]);
+          u[v][4 + e] = __uint_as_float(raw[j][v].b[e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          u[v][2 * e] = bf16_lo(raw[j][v].a[e]);
+          u[v][2 * e + 1] = bf16_hi(raw[j][v].a[e]);
+        }
+      }
+      if (PRE) {
+        const f32x4 p1a = sP1[0][g], p1b = sP1[1][g], p0a = sP0[0][g], p0b = sP0[1][g];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          u[v][e] = act ? fmaf(u[v][e], p1a[e], p0a[e]) : 0.f;
+          u[v][4 + e] = act ? fmaf(u[v][4 + e], p1b[e], p0b[e]) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += (p.kind == AERIS_NORM_RMS) ? u[v][e] * u[v][e] : u[v][e];
+    }
+    s = wave_sum(s);
+    float mean = 0.f, rstd;
+    if (p.kind == AERIS_NORM_RMS) {
+      rstd = rsqrtf(s * inv_d + p.eps);
+    } else {
+      mean = s * inv_d;
+      float qs = 0.f;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const bool act = FULL || (v * 64 + lane) * 8 < d;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float c = act ? u[v][e] - mean : 0.f;
+          qs += c * c;
+        }
+      }
+      qs = wave_sum(qs);
+      rstd = rsqrtf(qs * inv_d + p.eps);
+    }
+    if (row < end) {
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const int g = v * 64 + lane;
+        if (!(FULL || g * 8 < d)) continue;
+        const f32x4 ga = sG[0][g], gb = sG[1][g], ba = sB[0][g], bb = sB[1][g];
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o[e] = fmaf((u[v][e] - mean) * rstd, ga[e], ba[e]);
+          o[4 + e] = fmaf((u[v][4 + e] - mean) * rstd, gb[e], bb[e]);
+        }
+        if (p.y_dtype == AERIS_BF16) {
+          const u32x4 wv = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
+          __builtin_nontemporal_store(wv, (__attribute__((address_space(1))) u32x4*)(yg + (row * d + g * 8) * 2));
+        } else {
+          const g_ptr yp = yg + (row * d + g * 8) * 4;
+          __builtin_nontemporal_store(f32x4{o[0], o[1], o[2], o[3]}, (__attribute__((address_space(1))) f32x4*)yp);
+          __builtin_nontemporal_store(f32x4{o[4], o[5], o[6], o[7]}, (__attribute__((address_space(1))) f32x4*)(yp + 16));
+        }
+      }
+    }
+  }
+}
+
 bool norm_supported(int d) { return d > 0 && d % 8 == 0 && d <= 12 * 512; }
 
 template <int NV>
 static hipError_t launch_norm(const NormParams& p, bool x_f32, bool pre, hipStream_t stream) {
+  if constexpr (NV <= 4) {
+    // rows of up to 2048 elements: blocks of 4 waves x 2 rows that never straddle a batch entry
+    constexpr int ROWS = 2;
+    const int64_t rpb = p.mod_batch_stride ? p.rows_per_batch : p.rows;
+    const int64_t batches = (p.rows + rpb - 1) / rpb;
+    const int64_t bpb = (rpb + 4 * ROWS - 1) / (4 * ROWS);
+    if (batches * bpb >= (int64_t(1) << 31)) return hipErrorInvalidValue;
+    {
+      NormParams q = p;
+      q.rows_per_batch = rpb;
+      dim3 grid((unsigned)(batches * bpb)), block(256);
+#define AERIS_NORM_BLK(XF, PR)                                                                                           \
+  do {                                                                                                                   \
+    if (p.d == NV * 512)                                                                                                   \
+      hipLaunchKernelGGL((norm_modulate_block_kernel<NV, XF, PR, true, ROWS>), grid, block, 0, stream, q, bpb);                  \
+    else                                                                                                                   \
+      hipLaunchKernelGGL((norm_modulate_block_kernel<NV, XF, PR, false, ROWS>), grid, block, 0, stream, q, bpb);                 \
+  } while (0)
+      if (x_f32) {
+        if (pre) AERIS_NORM_BLK(true, true);
+        else AERIS_NORM_BLK(true, false);
+      } else {
+        if (pre) AERIS_NORM_BLK(false, true);
+        else AERIS_NORM_BLK(false, false);
+      }
+#undef AERIS_NORM_BLK
+      return hipGetLastError();
+    }
+  } else {
   // enough waves to cover HBM latency, few enough that parameter folding is amortised over many rows
   int64_t blocks = (p.rows + 3) / 4;
   const int64_t cap = 256 * 8;
@@ -198,6 +408,7 @@ static hipError_t launch_norm(const NormParams& p, bool x_f32, bool pre, hipStre
   }
 #undef AERIS_NORM_GO
   return hipGetLastError();
+  }
 }
 
 hipError_t norm_modulate_launch(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,

@@ -102,6 +102,7 @@ int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const vo
 /* Row norm fused with noise-level modulation.
  *   x  [B*rows_per_batch, d] (x_dtype bf16|f32)  ->  y [B*rows_per_batch, d] (y_dtype bf16|f32)
  *   gamma [d]; beta [d] or NULL (both param_dtype bf16|f32); shift, scale f32 [B_mod, d] or NULL
+ *   (gamma, beta, shift, scale 16-byte aligned and mod_batch_stride a multiple of 4: they are read 16 bytes at a time)
  *   (B_mod = 1 or B, given by mod_batch_stride: 0 = one row broadcast over the batch, otherwise the
  *   distance in elements between the rows of consecutive batch entries)
  * Replaces torch.nn.RMSNorm + modulate (model.py:121-125,400-401,426) / LayerNorm + modulate. */

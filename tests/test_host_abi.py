@@ -92,6 +92,9 @@ def test_argument_validation_needs_no_gpu(pkg):
     assert g(p16, 0, p16, 0, p16, None, 0, None, None, 0, 1, 4, 60, 0, 0, 1e-5, None) == L.EUNSUPPORTED  # d % 8
     assert g(p16, 7, p16, 0, p16, None, 0, None, None, 0, 1, 4, 64, 0, 0, 1e-5, None) == L.EINVAL  # dtype
     assert g(p16, 0, p16, 0, p16, None, 0, None, None, 0, 1, 4, 64, 5, 0, 1e-5, None) == L.EINVAL  # kind
+    assert g(p16, 0, p16, 0, p16 + 2, None, 0, None, None, 0, 1, 4, 64, 0, 0, 1e-5, None) == L.EINVAL  # gamma not 16-byte aligned
+    assert g(p16, 0, p16, 0, p16, None, 0, p16 + 4, None, 64, 1, 4, 64, 0, 0, 1e-5, None) == L.EINVAL  # shift not aligned
+    assert g(p16, 0, p16, 0, p16, None, 0, p16, p16, 66, 1, 4, 64, 0, 0, 1e-5, None) == L.EINVAL  # mod_batch_stride % 4
     # gemm
     h = lib.aeris_gemm_fwd
     assert h(p16, p16, p16, None, None, None, 8, 8, 100, 8, 0, 0, 0, 0, 0, None) == L.EUNSUPPORTED  # K % 64

@@ -1,7 +1,9 @@
 // Windowed multi-head self-attention for gfx950, streaming variant: windows of any size up to 4096 tokens
 // (the reference's 60 x 60) and head_dim 64 or 128, no relative-position bias, no shift mask (model.py:289-293).
 //
-// One workgroup = 128 queries of one (window, head): 4 waves x 32 queries.  The keys of the window are streamed
+// One workgroup = 256 queries of one (window, head): 8 waves x 32 queries, one workgroup per CU (with 128 queries per
+// workgroup and two workgroups per CU every K / V chunk was loaded, transposed and stored twice as often per query:
+// 6-7 % slower).  The keys of the window are streamed
 // through LDS in chunks of 64 (double buffered: the global loads of chunk j+1 are in flight while chunk j is
 // being consumed) with an online softmax (running row max m and row sum l, output rescaled only when a max
 // moves).  Window partition, window reverse and the cyclic shift are address arithmetic exactly as in the
@@ -35,7 +37,8 @@ struct StreamParams {
 };
 
 constexpr int KC = 64;    // keys per chunk
-constexpr int QB = 128;   // queries per workgroup
+constexpr int NWAVE = 8;         // waves per workgroup (two per SIMD, one workgroup per CU)
+constexpr int QB = 32 * NWAVE;   // queries per workgroup
 constexpr int MAX_L = 4096;
 
 // byte offset of 16-byte chunk `chunk` of row `row` in a tile with 128-byte rows (8 chunks), swizzled over double rows
@@ -67,14 +70,14 @@ struct StreamCfg {
 }  // namespace
 
 template <int HD>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(64 * NWAVE) __attribute__((amdgpu_waves_per_eu(2)))
 window_attention_stream_kernel(StreamParams p) {
   using Cfg = StreamCfg<HD>;
   constexpr int CH = HD / 8;   // 16-byte chunks per head row
   constexpr int KS = HD / 16;  // k16 steps of QK^T
   constexpr int DB = HD / 32;  // 32-row blocks of O^T
-  constexpr int NT = 256;
-  constexpr int KIT = KC * CH / NT;                     // 16-byte K pieces per thread and chunk (2 or 4)
+  constexpr int NT = 64 * NWAVE;
+  constexpr int KIT = KC * CH / NT;                     // 16-byte K pieces per thread and chunk (1 or 2)
   constexpr int V_ITEMS = (KC / 4) * CH;                // (4 keys x 8 d) V pieces per chunk: 128 or 256
   constexpr float LOG2E = 1.4426950408889634f;
 
@@ -128,7 +131,7 @@ window_attention_stream_kernel(StreamParams p) {
   const int nch = (L + KC - 1) / KC;
 
   u32x4 kreg[KIT], vreg[4];
-  const bool v_item = (V_ITEMS >= NT) || tid < V_ITEMS;  // head_dim 64: half of the threads carry a V piece
+  const bool v_item = (V_ITEMS >= NT) || tid < V_ITEMS;  // waves 0-3 (head_dim 64: waves 0-1) carry a V piece
   // V piece of this thread: 4 keys (key group v_kg of the chunk) x 8 d (piece v_c).  Lane bits 0-2 (and 4 for head_dim
   // 128) select the piece - the lanes of a key group still cover whole rows of V - bit 3 the key group within a pair
   // that shares a 16-byte chunk of V^T: see vt_off().
@@ -200,15 +203,20 @@ window_attention_stream_kernel(StreamParams p) {
   store_chunk(0);
   __syncthreads();
 
+  // A wave whose 32 queries all lie past the window (last query block of a window whose size is not a multiple of 256)
+  // only stages K / V and keeps the barriers; its MFMA and softmax work would be thrown away.
+  const bool wave_active = qb * QB + wave * 32 < L;  // wave-uniform
+
   for (int j = 0; j < nch; ++j) {
     if (j + 1 < nch) load_chunk(j + 1);
     const unsigned char* sK = smem + (j & 1) * Cfg::BUF;
     const unsigned char* sV = sK + Cfg::K_BYTES;
+    f32x16 acc[2];
+    if (wave_active) {
 
     // ---- S^T = K Q^T for the 64 keys of the chunk: acc[kb][4g+i] = <k[key], q>, key = 64j + 32kb + 8g + 4hi + i
     // The K fragments are read PF MFMAs ahead of their use (left to itself the compiler reads each one right before
     // its MFMA and exposes the LDS latency every time).
-    f32x16 acc[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -300,6 +308,7 @@ window_attention_stream_kernel(StreamParams p) {
       for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfb[step & 1][db], pf, o[db], 0, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
+    }  // wave_active
 
     if (j + 1 < nch) store_chunk((j + 1) & 1);
     __syncthreads();
@@ -356,9 +365,9 @@ hipError_t attention_stream_launch(const void* qkv, void* out, int B, int H, int
   const int64_t grid = (int64_t)((p.n_units + 7) / 8) * 8 * p.qblks;
   const int smem = stream_smem(head_dim, L);
   if (head_dim == 64)
-    hipLaunchKernelGGL(window_attention_stream_kernel<64>, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    hipLaunchKernelGGL(window_attention_stream_kernel<64>, dim3((unsigned)grid), dim3(64 * NWAVE), smem, stream, p);
   else
-    hipLaunchKernelGGL(window_attention_stream_kernel<128>, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    hipLaunchKernelGGL(window_attention_stream_kernel<128>, dim3((unsigned)grid), dim3(64 * NWAVE), smem, stream, p);
   return hipGetLastError();
 }
 

@@ -4,8 +4,8 @@
 // One workgroup = 256 queries of one (window, head): 8 waves x 32 queries, one workgroup per CU (with 128 queries per
 // workgroup and two workgroups per CU every K / V chunk was loaded, transposed and stored twice as often per query:
 // 6-7 % slower).  The keys of the window are streamed
-// through LDS in chunks of 64 (double buffered: the global loads of chunk j+1 are in flight while chunk j is
-// being consumed) with an online softmax (running row max m and row sum l, output rescaled only when a max
+// through LDS in chunks of 64 (four buffers: the global loads of chunk j+2 are in flight while chunk j is
+// being consumed, and are written to LDS at its end) with an online softmax (running row max m and row sum l, output rescaled only when a max
 // moves).  Window partition, window reverse and the cyclic shift are address arithmetic exactly as in the
 // one-window-per-workgroup kernel (window_attention.hip); the token row of every window position is computed once
 // per workgroup into an LDS table, so the streaming loop needs no integer division.
@@ -40,6 +40,9 @@ constexpr int KC = 64;    // keys per chunk
 constexpr int NWAVE = 8;         // waves per workgroup (two per SIMD, one workgroup per CU)
 constexpr int QB = 32 * NWAVE;   // queries per workgroup
 constexpr int MAX_L = 4096;
+// K / V chunk buffers in LDS.  With four, chunk j + 2 is written while chunk j is consumed and the workgroup needs a
+// barrier only after every second chunk (2 buffers, one barrier per chunk: 2.5 % slower).
+constexpr int NBUF = 4;
 
 // byte offset of 16-byte chunk `chunk` of row `row` in a tile with 128-byte rows (8 chunks), swizzled over double rows
 __device__ __forceinline__ uint32_t off128(int row, int chunk) {
@@ -64,7 +67,7 @@ struct StreamCfg {
   static constexpr int K_BYTES = KC * HD * 2;
   static constexpr int V_BYTES = HD * KC * 2;
   static constexpr int BUF = K_BYTES + V_BYTES;
-  static constexpr int TBL_OFF = 2 * BUF;
+  static constexpr int TBL_OFF = NBUF * BUF;
 };
 
 }  // namespace
@@ -201,6 +204,10 @@ window_attention_stream_kernel(StreamParams p) {
 
   load_chunk(0);
   store_chunk(0);
+  if (NBUF == 4 && nch > 1) {
+    load_chunk(1);
+    store_chunk(1);
+  }
   __syncthreads();
 
   // A wave whose 32 queries all lie past the window (last query block of a window whose size is not a multiple of 256)
@@ -208,8 +215,9 @@ window_attention_stream_kernel(StreamParams p) {
   const bool wave_active = qb * QB + wave * 32 < L;  // wave-uniform
 
   for (int j = 0; j < nch; ++j) {
-    if (j + 1 < nch) load_chunk(j + 1);
-    const unsigned char* sK = smem + (j & 1) * Cfg::BUF;
+    constexpr int LEAD = NBUF / 2;  // chunk j + LEAD is loaded and written to LDS while chunk j is consumed
+    if (j + LEAD < nch) load_chunk(j + LEAD);
+    const unsigned char* sK = smem + (j & (NBUF - 1)) * Cfg::BUF;
     const unsigned char* sV = sK + Cfg::K_BYTES;
     f32x16 acc[2];
     if (wave_active) {
@@ -310,8 +318,8 @@ window_attention_stream_kernel(StreamParams p) {
     __builtin_amdgcn_sched_barrier(0);
     }  // wave_active
 
-    if (j + 1 < nch) store_chunk((j + 1) & 1);
-    __syncthreads();
+    if (j + LEAD < nch) store_chunk((j + LEAD) & (NBUF - 1));
+    if (NBUF == 2 || (j & 1)) __syncthreads();
   }
 
   // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i]
@@ -333,7 +341,7 @@ window_attention_stream_kernel(StreamParams p) {
 
 // ---------------------------------------------------------------------------------------------
 
-static int stream_smem(int head_dim, int L) { return 2 * (KC * head_dim * 2 + head_dim * KC * 2) + ((L * 4 + 15) / 16) * 16; }
+static int stream_smem(int head_dim, int L) { return NBUF * (KC * head_dim * 2 + head_dim * KC * 2) + ((L * 4 + 15) / 16) * 16; }
 
 bool attention_stream_supported(int ws_y, int ws_x, int head_dim, bool has_bias, bool use_mask) {
   const int64_t L = (int64_t)ws_y * ws_x;

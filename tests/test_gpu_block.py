@@ -229,3 +229,29 @@ def test_full_grid_ensemble_batch_matches_single_members(pkg, cuda):
             torch.cuda.synchronize()
             assert torch.equal(out[b:b + 1], single), (shifted, b)
         assert bool(torch.isfinite(out.float()).all())
+
+
+@pytest.mark.gpu
+def test_bench_json_contract_on_a_small_workload(pkg, cuda, monkeypatch, capsys):
+    """bench.py's one JSON line carries the fields its callers read (run in-process on the configs[1] shape: seconds)."""
+    import json
+    import sys
+    import bench
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--workload", "config1", "--steps", "1", "--warmup", "0", "--cpu-rows", "12"])
+    bench.main()
+    line = [l for l in capsys.readouterr().out.strip().splitlines() if l.startswith("{")][-1]
+    r = json.loads(line)
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "kernels", "cpu_baseline"):
+        assert key in r, key
+    assert r["n_gpus"] == 1 and r["steps"] == 1 and r["higher_is_better"] is True and r["vs_baseline"] is None
+    assert r["value"] > 0 and abs(r["value"] * r["ms_per_step"] - 1000.0) < 1e-6 * 1000.0
+    assert "workload" in r["config"] and "model" not in r["config"]
+    assert r["output_finite"] is True
+    cb = r["cpu_baseline"]
+    assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and "sample" in cb
+    if r["roofline"] is not None:
+        rf = r["roofline"]
+        assert rf["bound"] in ("hbm", "mfma") and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
+    for k in r["kernels"].values():
+        assert k["launches_per_step"] >= 1 and k["avg_ms"] > 0

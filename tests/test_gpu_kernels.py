@@ -89,6 +89,28 @@ def test_gemm_parity(pkg, cuda, case):
     assert torch.isfinite(out).all()
 
 
+def test_gemm_gelu_epilogue_pointwise(pkg, cuda):
+    """The GELU of the GEMM epilogue, value by value: with one non-zero column in A and ones in W every output is
+    GELU(x) for a chosen x.  Against the erf form in float64: the epilogue's polynomial is within 2.1e-4 |x| (a tenth of
+    half a bf16 ulp; beyond |x| = 3.5 this is the clamp's 1 - Phi(3.5)) before the result is rounded to bf16."""
+    M, N, K = 8192, 256, 64
+    x = bf(torch.cat([torch.linspace(-8, 8, M - 2048), torch.linspace(-0.05, 0.05, 2048)]))
+    a = torch.zeros(M, K, dtype=torch.bfloat16)
+    a[:, 0] = x
+    w = torch.zeros(N, K, dtype=torch.bfloat16)
+    w[:, 0] = 1.0
+    out = pkg.ops.gemm(a.to(cuda), w.to(cuda), None, act="gelu").float().cpu()
+    xd = x.double()
+    exact = 0.5 * xd * (1.0 + torch.erf(xd / math.sqrt(2.0)))
+    bound = 2.1e-4 * xd.abs() + 2.0 ** -8 * exact.abs() + 1e-30
+    err = (out.double() - exact[:, None]).abs()
+    assert bool((err <= bound[:, None]).all()), float((err / bound[:, None]).max())
+    assert torch.equal(out, out[:, :1].expand_as(out))  # every column took the same path
+    # where the values are not small against |x| (x >= -1): within one bf16 ulp of the exact value
+    core = xd >= -1
+    assert bool((err[core] <= 2.0 ** -7 * exact[core].abs()[:, None] + 1e-30).all())
+
+
 def test_gemm_residual_in_place_and_deterministic(pkg, cuda):
     g = torch.Generator().manual_seed(0)
     a, w = bf(torch.randn(5000, 256, generator=g)).to(cuda), bf(torch.randn(384, 256, generator=g) / 16).to(cuda)

@@ -27,8 +27,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Bytes that crossed the L2 <-> fabric boundary per launch at the config3 workload (average over the launches of
 # one step), from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a 1 GiB copy kernel; the summary
 # with the commands is profiles/denoiser_step_config3_pmc_traffic.txt.  Not measurable from inside this script.
-PMC_TRAFFIC_BYTES = {"config3": {"gemm_256x256_none_bf16_res": 33.087e9 + 3.185e9, "gemm_256x256_none_bf16_plain": 31.001e9 + 9.300e9,
-                                 "gemm_256x256_gelu_bf16_plain": 32.891e9 + 12.740e9,
+PMC_TRAFFIC_BYTES = {"config3": {"gemm_256x256_none_bf16_res": 33.650e9 + 3.185e9, "gemm_256x256_none_bf16_plain": 31.879e9 + 9.300e9,
+                                 "gemm_256x256_gelu_bf16_plain": 32.937e9 + 12.740e9,
                                  "window_attention": 9.556e9 + 3.185e9, "norm_modulate": 3.185e9 + 3.185e9}}
 
 WORKLOADS = {

@@ -38,8 +38,9 @@ SIGNATURES = {
     "aeris_gemm_heads_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_int, _c_i64, _c_vp]),
     "aeris_modulation_linear_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_vp]),
     "aeris_timestep_embedding_fwd": (_c_int, [_c_vp, _c_vp, _c_int, _c_int, _c_f32, _c_vp]),
-    "aeris_embed_prepare_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
-    "aeris_embed_concat_fwd": (_c_int, [_c_vp, _c_int, _c_f32, _c_vp, _c_int, _c_vp, _c_vp, _c_i64, _c_i64, _c_int, _c_vp]),
+    "aeris_embed_prepare_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_vp]),
+    "aeris_embed_concat_fwd": (_c_int, [_c_vp, _c_int, _c_f32, _c_vp, _c_int, _c_vp, _c_vp, _c_i64, _c_i64, _c_int, _c_int,
+                                        _c_vp]),
 }
 
 _lib = None

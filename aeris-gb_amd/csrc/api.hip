@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdarg>
 #include <cstdio>
+#include <atomic>
 #include <mutex>
 
 #include "kernels.h"
@@ -24,13 +25,23 @@ int hip_fail(hipError_t e, const char* what) {
 }
 
 std::once_flag g_init_once;
+std::atomic<bool> g_init_done{false};
 hipError_t g_init_status = hipSuccess;
 
-int ensure_init() {
+// One-time kernel attribute set-up.  A launch entry point performs it lazily, but never inside a stream capture:
+// hipFuncSetAttribute is not a stream operation and must not run while `stream` is being recorded into a graph.
+int ensure_init(void* stream = nullptr, bool from_launch = false) {
+  if (from_launch && !g_init_done.load(std::memory_order_acquire)) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(reinterpret_cast<hipStream_t>(stream), &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+      return fail(AERIS_EINVAL, "the library is not initialised and the stream is being captured: call aeris_init() "
+                                "before the capture begins");
+  }
   std::call_once(g_init_once, [] {
     g_init_status = aeris::gemm_configure_all();
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_configure_all();
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_stream_configure_all();
+    g_init_done.store(true, std::memory_order_release);
   });
   if (g_init_status != hipSuccess) return hip_fail(g_init_status, "aeris_init (hipFuncSetAttribute)");
   return AERIS_OK;
@@ -132,7 +143,7 @@ static int window_attention_impl(const char* who, const void* qkv, void* out, co
   const int64_t units = (int64_t)B * (H / ws_y) * (W / ws_x) * heads;
   if (units > 0x7fffffffLL || (!small && (units + 8) * (((int64_t)ws_y * ws_x + 127) / 128) > 0x7fffffffLL))
     return fail(AERIS_EUNSUPPORTED, "%s: more than 2^31-1 workgroups", who);
-  if (int rc = ensure_init()) return rc;
+  if (int rc = ensure_init(stream, true)) return rc;
   if (!small) {
     hipError_t e = aeris::attention_stream_launch(qkv, out, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x, scale,
                                                   tok_stride, head_stride, part_stride, reinterpret_cast<hipStream_t>(stream));
@@ -204,7 +215,7 @@ int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, cons
     return fail(AERIS_EINVAL, "aeris_gemm_fwd: rows_per_batch must be positive with a per-batch gate");
   if (gate_batch_stride < 0) return fail(AERIS_EINVAL, "aeris_gemm_fwd: negative gate_batch_stride");
   if ((int64_t)((M + 127) / 128) * ((N + 63) / 64) > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_fwd: too many tiles");
-  if (int rc = ensure_init()) return rc;
+  if (int rc = ensure_init(stream, true)) return rc;
   hipError_t e = aeris::gemm_launch(A, W, C, bias, gate, residual, M, N, K, ldc, act, res_dtype, c_dtype,
                                     gate_batch_stride, rows_per_batch, 0, 0, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_gemm_fwd launch");
@@ -222,7 +233,7 @@ int aeris_gemm_heads_fwd(const void* A, const void* W, void* C, const void* bias
   if (plane_stride < M * head_dim || plane_stride % 8)
     return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: plane_stride must be a multiple of 8 and at least M * head_dim");
   if ((int64_t)((M + 127) / 128) * ((N + 63) / 64) > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_heads_fwd: too many tiles");
-  if (int rc = ensure_init()) return rc;
+  if (int rc = ensure_init(stream, true)) return rc;
   hipError_t e = aeris::gemm_launch(A, W, C, bias, nullptr, nullptr, M, N, K, N, AERIS_ACT_NONE, -1, AERIS_BF16, 0, M, head_dim,
                                     plane_stride, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_gemm_heads_fwd launch");
@@ -252,26 +263,27 @@ int aeris_timestep_embedding_fwd(const float* t, float* emb, int B, int dim, flo
 }
 
 int aeris_embed_prepare_fwd(const float* x, const float* ape, void* out, int64_t M, int64_t M_ape, int C, int K_pad,
-                            void* stream) {
+                            int split, void* stream) {
   if (!x || !out) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: x/out is NULL");
-  if (M <= 0 || C <= 0 || K_pad < C || K_pad % 64) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: need M > 0, 0 < C <= K_pad, K_pad %% 64 == 0");
+  if (M <= 0 || C <= 0 || K_pad < (split ? 3 * (int64_t)C + 2 : (int64_t)C) || K_pad % 64)
+    return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: need M > 0, C > 0, K_pad >= C (3 C + 2 with split), K_pad %% 64 == 0");
   if (ape && M_ape <= 0) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: M_ape must be positive when ape is given");
   if (!aligned16(out)) return fail(AERIS_EINVAL, "aeris_embed_prepare_fwd: out must be 16-byte aligned");
-  hipError_t e = aeris::embed_prepare_launch(x, C, 1.0f, nullptr, 0, ape, out, M, M_ape > 0 ? M_ape : 1, K_pad,
+  hipError_t e = aeris::embed_prepare_launch(x, C, 1.0f, nullptr, 0, ape, out, M, M_ape > 0 ? M_ape : 1, K_pad, split,
                                              reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_embed_prepare_fwd launch");
   return AERIS_OK;
 }
 
 int aeris_embed_concat_fwd(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
-                           int64_t M, int64_t M_ape, int K_pad, void* stream) {
+                           int64_t M, int64_t M_ape, int K_pad, int split, void* stream) {
   if (!x0 || !x1 || !out) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: x0/x1/out is NULL");
-  if (M <= 0 || C0 <= 0 || C1 <= 0 || K_pad < C0 + C1 || K_pad % 64)
-    return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: need M > 0, C0 > 0, C1 > 0, C0 + C1 <= K_pad, K_pad %% 64 == 0");
+  if (M <= 0 || C0 <= 0 || C1 <= 0 || K_pad < (split ? 3 * ((int64_t)C0 + C1) + 2 : (int64_t)C0 + C1) || K_pad % 64)
+    return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: need M > 0, C0 > 0, C1 > 0, K_pad >= C0 + C1 (3 (C0 + C1) + 2 with split), K_pad %% 64 == 0");
   if (!(div0 != 0.0f)) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: div0 must be non-zero");
   if (ape && M_ape <= 0) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: M_ape must be positive when ape is given");
   if (!aligned16(out)) return fail(AERIS_EINVAL, "aeris_embed_concat_fwd: out must be 16-byte aligned");
-  hipError_t e = aeris::embed_prepare_launch(x0, C0, div0, x1, C1, ape, out, M, M_ape > 0 ? M_ape : 1, K_pad,
+  hipError_t e = aeris::embed_prepare_launch(x0, C0, div0, x1, C1, ape, out, M, M_ape > 0 ? M_ape : 1, K_pad, split,
                                              reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_embed_concat_fwd launch");
   return AERIS_OK;

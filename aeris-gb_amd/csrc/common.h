@@ -62,16 +62,19 @@ __device__ __forceinline__ float erf_poly(float x) {
 }
 __device__ __forceinline__ float gelu_erf_f(float x) { return 0.5f * x * (1.0f + erf_poly(x * 0.70710678118654752440f)); }
 
-// erf-GELU for results that are rounded to bf16: GELU(x) = x * (0.5 + t * P(t^2)), t = clamp(x, -3.5, 3.5),
+// erf-GELU for results that are rounded to bf16: GELU(x) = xm * (0.5 + t * P(t^2)), xm = max(x, -3.5), t = min(xm, 3.5),
 // t * P(t^2) = erf(t / sqrt2) / 2 with P a degree-6 minimax polynomial for the error measure |GELU error| / |x| (the
-// 1/sqrt2 and the 1/2 are folded into its coefficients): |error| <= 2.0e-4 |x| everywhere, a tenth of half a bf16 ulp,
-// the clamp included (1 - Phi(3.5) = 2.3e-4).  On normally distributed inputs 2 % of the bf16 results differ by one ulp
-// from the exactly evaluated and once-rounded GELU (0.7 % for a 1.5e-7 evaluation: rounding an fp32 result to bf16
-// twice), the relative L2 error after rounding is the same to four digits.  10 VALU operations and no
-// transcendental, against about 24 op-equivalents for the 1.5e-7 version above and 12 for a degree-8 polynomial over
-// +-3 sqrt2 (1.6e-5 |x|): the GEMM epilogue is VALU-bound, every two operations are worth 1.3 % of the fc1 GEMM.
+// 1/sqrt2 and the 1/2 are folded into its coefficients): |error| <= 2.0e-4 |x| for x >= -3.5, a tenth of half a bf16 ulp,
+// the clamp included (1 - Phi(3.5) = 2.3e-4); below -3.5 the result is the constant -3.5 * 2.3e-4 = -8.1e-4 where the
+// exact value decays from -8.1e-4 to 0, so large negative pre-activations cannot leak a term proportional to x.
+// On normally distributed inputs 2 % of the bf16 results differ by one ulp from the exactly evaluated and
+// once-rounded GELU (0.7 % for a 1.5e-7 evaluation: rounding an fp32 result to bf16 twice), the relative L2 error
+// after rounding is the same to four digits.  11 VALU operations and no transcendental, against about 24
+// op-equivalents for the 1.5e-7 version above and 12 for a degree-8 polynomial over +-3 sqrt2 (1.6e-5 |x|): the GEMM
+// epilogue is VALU-bound, every two operations are worth 1.3 % of the fc1 GEMM.
 __device__ __forceinline__ float gelu_bf16_f(float x) {
-  const float t = __builtin_amdgcn_fmed3f(x, -3.5f, 3.5f);
+  const float xm = fmaxf(x, -3.5f);
+  const float t = fminf(xm, 3.5f);
   const float s = t * t;
   float p = fmaf(5.387934375e-08f, s, -2.947825681e-06f);
   p = fmaf(p, s, 7.079321479e-05f);
@@ -79,7 +82,7 @@ __device__ __forceinline__ float gelu_bf16_f(float x) {
   p = fmaf(p, s, 9.561960235e-03f);
   p = fmaf(p, s, -6.607216932e-02f);
   p = fmaf(p, s, 3.988177931e-01f);
-  return x * fmaf(t, p, 0.5f);
+  return xm * fmaf(t, p, 0.5f);
 }
 
 }  // namespace aeris

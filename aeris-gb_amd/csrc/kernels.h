@@ -37,7 +37,6 @@ hipError_t modulation_linear_launch(const float* x, const void* W, const void* b
                                     int w_dtype, int act, hipStream_t stream);
 hipError_t timestep_embedding_launch(const float* t, float* emb, int B, int dim, float max_period, hipStream_t stream);
 hipError_t embed_prepare_launch(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
-                                int64_t M, int64_t M_ape, int K_pad,
-                                hipStream_t stream);
+                                int64_t M, int64_t M_ape, int K_pad, int split, hipStream_t stream);
 
 }  // namespace aeris

@@ -86,8 +86,13 @@ hipError_t timestep_embedding_launch(const float* t, float* emb, int B, int dim,
   return hipGetLastError();
 }
 
-// out[m, k] = bf16(x[m, k] + ape[m % M_ape, k]) for k < C, 0 for C <= k < K_pad.  One thread per 8 output columns.
-// out[m, :] = [x0[m, :] / div0 | x1[m, :]] + ape[m % M_ape, :], zero padded to K_pad columns (x1 may be absent)
+// out[m, :] = [x0[m, :] / div0 | x1[m, :]] + ape[m % M_ape, :] as bf16, zero padded to K_pad columns (x1 may be
+// absent).  One thread per 8 output columns.
+// SPLIT: the C values v are written three times and followed by two ones, [hi | lo | hi | 1 | 1] with hi = bf16(v),
+// lo = bf16(v - hi); against a weight matrix laid out [W_hi | W_hi | W_lo | b_hi | b_lo] the bf16 GEMM then returns
+// v W^T + b to about 2^-16 relative (hi W_hi + lo W_hi + hi W_lo; only lo W_lo is dropped), which is what keeps the
+// embedding at the accuracy of the reference's fp32 Linear.
+template <bool SPLIT>
 __global__ void __launch_bounds__(256) embed_prepare_kernel(const float* __restrict__ x0, int C0, float div0,
                                                            const float* __restrict__ x1, int C1,
                                                            const float* __restrict__ ape, uint16_t* __restrict__ out,
@@ -104,11 +109,18 @@ __global__ void __launch_bounds__(256) embed_prepare_kernel(const float* __restr
   float v[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const int k = k0 + e;
+    int k = k0 + e;
+    bool lo = false;
     v[e] = 0.f;
+    if (SPLIT) {
+      if (k >= 3 * C) { if (k < 3 * C + 2) v[e] = 1.f; k = C; }
+      else if (k >= 2 * C) k -= 2 * C;
+      else if (k >= C) { k -= C; lo = true; }
+    }
     if (k < C) {
       const float xv = k < C0 ? (div0 == 1.0f ? r0[k] : r0[k] / div0) : r1[k - C0];
-      v[e] = xv + (ar ? ar[k] : 0.f);
+      const float val = xv + (ar ? ar[k] : 0.f);
+      v[e] = lo ? val - bf16_bits_to_f32(f32_to_bf16_bits(val)) : val;
     }
   }
   u32x4 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
@@ -116,10 +128,15 @@ __global__ void __launch_bounds__(256) embed_prepare_kernel(const float* __restr
 }
 
 hipError_t embed_prepare_launch(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
-                                int64_t M, int64_t M_ape, int K_pad, hipStream_t stream) {
+                                int64_t M, int64_t M_ape, int K_pad, int split, hipStream_t stream) {
   const int64_t n = M * (K_pad / 8);
-  hipLaunchKernelGGL(embed_prepare_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x0, C0, div0, x1, C1,
-                     ape, reinterpret_cast<uint16_t*>(out), M, M_ape, K_pad);
+  const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (split)
+    hipLaunchKernelGGL(embed_prepare_kernel<true>, grid, block, 0, stream, x0, C0, div0, x1, C1, ape,
+                       reinterpret_cast<uint16_t*>(out), M, M_ape, K_pad);
+  else
+    hipLaunchKernelGGL(embed_prepare_kernel<false>, grid, block, 0, stream, x0, C0, div0, x1, C1, ape,
+                       reinterpret_cast<uint16_t*>(out), M, M_ape, K_pad);
   return hipGetLastError();
 }
 

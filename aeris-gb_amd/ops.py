@@ -58,6 +58,7 @@ def gemm_uses_big_tiles(M, N, act=None):
 
 
 _WORKSPACE = {}
+_WS_OWNER = {}  # key -> the stream whose work last used the buffer
 _RETIRED = []  # outgrown buffers stay allocated: a captured HIP graph may still point into them
 
 
@@ -65,11 +66,27 @@ def workspace(tag: str, shape, dtype, device) -> torch.Tensor:
     """Reusable scratch tensor for an intermediate that never leaves the block (normalised tokens, qkv, attention
     output, MLP hidden).  One buffer per (tag, device, dtype), grown on demand and never freed, so eager calls and
     captured graphs share it instead of each holding a pool of their own (at batch 4 on the 720x1440 grid the four
-    intermediates are 115 GB).  Calls that use the same tag must be ordered on one stream."""
+    intermediates are 115 GB).
+
+    Every model, layer and captured graph on the device shares these buffers, which is safe as long as their uses are
+    ordered on one stream.  The buffer remembers the stream that used it last: a request from another stream is
+    accepted only when that stream has no work pending (then the buffer changes hands), otherwise two streams would be
+    writing one scratch area at the same time and this raises instead.  Calls made while a stream is being captured
+    are not checked, and replays of a captured graph do not pass through here: a graph must not be replayed on one
+    stream while model calls run on another."""
     n = 1
     for d in shape:
         n *= int(d)
     key = (tag, str(device), dtype)
+    if not torch.cuda.is_current_stream_capturing():
+        # (a capture queues no work and nothing may be queried while it runs: it neither checks nor takes the buffer)
+        cur = torch.cuda.current_stream(device)
+        owner = _WS_OWNER.get(key)
+        if owner is not None and owner != cur and not owner.query():
+            raise RuntimeError(f"workspace {tag!r} on {device} is in use by work pending on another stream: the block "
+                               "intermediates are shared per device, run the models of one device on one stream "
+                               "(or synchronise the other stream first)")
+        _WS_OWNER[key] = cur
     buf = _WORKSPACE.get(key)
     if buf is None or buf.numel() < n:
         if buf is not None:
@@ -308,8 +325,9 @@ def timestep_embedding(t: torch.Tensor, dim: int, max_period: float = 10_000.0,
     return out
 
 
-def embed_prepare(x: torch.Tensor, ape: Optional[torch.Tensor], k_pad: int, out: Optional[torch.Tensor] = None):
-    """bf16 [M, k_pad] = x f32 [M, C] (+ ape f32 [M_ape, C], row m % M_ape), zero padded."""
+def embed_prepare(x: torch.Tensor, ape: Optional[torch.Tensor], k_pad: int, out: Optional[torch.Tensor] = None,
+                  split: bool = False):
+    """bf16 [M, k_pad] = x f32 [M, C] (+ ape f32 [M_ape, C], row m % M_ape), zero padded; ``split``: [hi | lo | hi]."""
     _dev(x, "x", torch.float32)
     C = x.shape[-1]
     M = x.numel() // C
@@ -321,13 +339,14 @@ def embed_prepare(x: torch.Tensor, ape: Optional[torch.Tensor], k_pad: int, out:
             raise RuntimeError("ape must be [M_ape, C] with M a multiple of M_ape")
     if out is None:
         out = torch.empty(M, k_pad, dtype=torch.bfloat16, device=x.device)
-    L.call("aeris_embed_prepare_fwd", x.data_ptr(), _ptr(ape), out.data_ptr(), M, m_ape, C, k_pad, _stream())
+    L.call("aeris_embed_prepare_fwd", x.data_ptr(), _ptr(ape), out.data_ptr(), M, m_ape, C, k_pad, int(split), _stream())
     return out
 
 
 def embed_concat(x0: torch.Tensor, div0: float, x1: torch.Tensor, ape: Optional[torch.Tensor], k_pad: int,
-                 out: Optional[torch.Tensor] = None):
-    """bf16 [M, k_pad] = [x0 f32 [M, C0] / div0 | x1 f32 [M, C1]] (+ ape f32 [M_ape, C0 + C1]), zero padded."""
+                 out: Optional[torch.Tensor] = None, split: bool = False):
+    """bf16 [M, k_pad] = [x0 f32 [M, C0] / div0 | x1 f32 [M, C1]] (+ ape f32 [M_ape, C0 + C1]), zero padded;
+    ``split``: the values three times as [hi | lo | hi]."""
     _dev(x0, "x0", torch.float32)
     _dev(x1, "x1", torch.float32)
     C0, C1 = x0.shape[-1], x1.shape[-1]
@@ -343,5 +362,5 @@ def embed_concat(x0: torch.Tensor, div0: float, x1: torch.Tensor, ape: Optional[
     if out is None:
         out = torch.empty(M, k_pad, dtype=torch.bfloat16, device=x0.device)
     L.call("aeris_embed_concat_fwd", x0.data_ptr(), C0, float(div0), x1.data_ptr(), C1, _ptr(ape), out.data_ptr(), M,
-           m_ape, k_pad, _stream())
+           m_ape, k_pad, int(split), _stream())
     return out

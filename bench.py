@@ -96,16 +96,18 @@ def run_rollout(args, pkg, torch, wl, model, dev):
         del x
     smp = pkg.TrigFlowSampler(model, n_steps=args.sampler_steps, device=dev)
     state0 = torch.randn(B, S, C, generator=g, device=dev)
-    smp.capture(state0, torch.randn(B, S, C, generator=g, device=dev), warmup=1)
     nfe = 2 * args.sampler_steps - 1
-    for _ in range(args.warmup):
-        smp.rollout(state0, 1, g, use_graph=True)
+    # one HIP graph = one whole forecast step: latent draw, 2n-1 denoiser calls, un-standardise + accumulate +
+    # re-standardise of the state; captured once, replayed per step
+    ro = smp.begin_rollout(state0, max(args.steps, args.warmup, 1), g, use_graph=True, graph_warmup=0)
+    ro.run(args.warmup)
+    ro.reset()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    states = smp.rollout(state0, args.steps, g, use_graph=True)
+    states = ro.run(args.steps)[:args.steps]
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    finite = all(bool(torch.isfinite(s_).all()) for s_ in states)
+    finite = bool(torch.isfinite(states).all())
     done.set()
     agg = {}
     for tag, work, unit, ms in rec:
@@ -167,7 +169,8 @@ def main():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
-    ap.add_argument("--residual", default="bf16", choices=["bf16", "f32"])
+    ap.add_argument("--residual", default="f32", choices=["bf16", "f32"],
+                    help="dtype of the residual stream between blocks (f32: within 1e-2 of fp32 at 24 blocks; bf16: not)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=96)
     ap.add_argument("--copy-calibration", action="store_true",

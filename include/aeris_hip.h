@@ -46,7 +46,7 @@ extern "C" {
 
 /* GEMM epilogue activations (aeris_gemm_fwd) */
 #define AERIS_ACT_NONE 0
-#define AERIS_ACT_GELU 1   /* exact erf GELU */
+#define AERIS_ACT_GELU 1   /* erf GELU 0.5 x (1 + erf(x / sqrt 2)), see the note at aeris_gemm_fwd */
 #define AERIS_ACT_SWIGLU 2 /* W has 2*N rows [gate | up]; C = silu(gate)*up  (model.py:156-158) */
 #define AERIS_ACT_SILU 3
 
@@ -117,7 +117,13 @@ int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, co
  *   gate f32 [B_mod, N] or NULL (gate_batch_stride as above, rows_per_batch rows of C per batch entry)
  *   residual [M, N] (res_dtype) or NULL, may alias C;  C [M, ldc] (c_dtype), ldc >= N
  * Replaces nn.Linear at model.py:153-154,284-285,342,418 and the gate/residual elementwise passes
- * at model.py:400-401.  Requires K % 64 == 0. */
+ * at model.py:400-401.  Requires K % 64 == 0.
+ * AERIS_ACT_GELU is the erf form in both tile kernels, evaluated to the accuracy of the output type.  bf16 C from
+ * the 256x256-tile kernel (M >= 256 and at least 256 tiles, N a multiple of 256 or >= 1024): a polynomial on the
+ * clamp [-3.5, 3.5], |error| <= 2.0e-4 |x| for x >= -3.5 (a tenth of half a bf16 ulp) and the constant -8.1e-4 below
+ * -3.5, where the exact value lies between -8.1e-4 and 0.  Every other case (f32 C, or the 128x128-tile kernel that
+ * takes small and ragged problems): erf to 1.5e-7 absolute.  The two agree to within one bf16 ulp of the result for
+ * x >= -1; which one runs depends on the shape only, never on the data. */
 int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, const float* gate,
                    const void* residual, int64_t M, int N, int K, int64_t ldc, int act, int res_dtype,
                    int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, void* stream);
@@ -138,16 +144,19 @@ int aeris_modulation_linear_fwd(const float* x, const void* W, const void* bias,
 int aeris_timestep_embedding_fwd(const float* t, float* emb, int B, int dim, float max_period, void* stream);
 
 /* A-operand preparation for the input embedding: out bf16 [M, K_pad] = (x f32 [M, C] + ape f32 [M_ape, C] or NULL),
- * zero padded from C to K_pad columns; ape row = m % M_ape.  (model.py:350-352) */
+ * zero padded from C to K_pad columns; ape row = m % M_ape.  (model.py:350-352)
+ * split != 0: the C values v are written as [hi | lo | hi | 1 | 1], hi = bf16(v), lo = bf16(v - hi), zero padded from
+ * 3 C + 2 to K_pad columns.  With the weight laid out [W_hi | W_hi | W_lo | b_hi | b_lo] along K the bf16 GEMM returns
+ * v W^T + b to about 2^-16 relative: the reference computes this Linear in fp32 (model.py:352). */
 int aeris_embed_prepare_fwd(const float* x, const float* ape, void* out, int64_t M, int64_t M_ape, int C,
-                            int K_pad, void* stream);
+                            int K_pad, int split, void* stream);
 
 /* The same with the sampler's channel concatenation folded in: out bf16 [M, K_pad] =
  * ([x0 f32 [M, C0] / div0 | x1 f32 [M, C1]] + ape f32 [M_ape, C0 + C1] or NULL), zero padded.  x0 is the noised state
  * (divided by sigma_data), x1 the conditioning channels: torch.cat([x_t / sigma_d, conditioning], dim=2) of
  * inference.py:160 followed by model.py:350-352, without materialising the concatenated tensor. */
 int aeris_embed_concat_fwd(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
-                           int64_t M, int64_t M_ape, int K_pad, void* stream);
+                           int64_t M, int64_t M_ape, int K_pad, int split, void* stream);
 
 #ifdef __cplusplus
 }

@@ -38,26 +38,46 @@ def sample(denoiser, cond, latents, t_steps, sigma_data=1.0):
     return x
 
 
-def rollout(denoiser, state0, n_forecast, n_diffusion, generator, sigma_min=0.2, sigma_max=500.0,
-            sigma_data=1.0, x_mean=None, x_std=None, t_mean=None, t_std=None, extra_cond=None):
-    """Autoregressive forecast: X <- X + unstd_t(sample); cond <- std_x(X)  (inference.py:180-186).
+def rollout(denoiser, state0, n_forecast, n_diffusion, generator=None, sigma_min=0.2, sigma_max=500.0,
+            sigma_data=1.0, x_mean=None, x_std=None, t_mean=None, t_std=None, forcing=None, static=None,
+            extra_cond=None, latents=None):
+    """Autoregressive forecast (inference.py:127-186).
 
-    ``state0`` is the standardised state ``[B, S, C]``.  Means/stds default to 0/1 (identity).
+    Per forecast step k the conditioning is ``cat([state, forcing[k], static, forcing[k+1], extra])`` along the
+    channels (inference.py:133: ``cat([condition, rad_T[k], gp, lsm, rad_T[k+1]])`` with forcing = rad_T and
+    static = cat([gp, lsm])); then ``X <- X + unstandardize_t(sample)`` and ``state <- standardize_x(X)``
+    (inference.py:180-186; era5.py:95-114: standardise = (x - mean) / std, un-standardise = x * std + mean).
+    ``state0`` is the standardised state ``[B, S, C]``; means / stds default to 0 / 1; ``forcing``
+    ``[n_forecast + 1, 1|B, S, Cf]``; ``static`` ``[1|B, S, Cs]``; ``extra_cond`` ``[1|B, S, Ce]`` or one per step
+    ``[n_forecast, 1|B, S, Ce]``; ``latents`` ``[n_forecast, B, S, C]`` replaces the draws from ``generator``.
     Returns the list of standardised states after every forecast step.
     """
-    C = state0.shape[-1]
+    B, _, C = state0.shape
     one, zero = torch.ones(C), torch.zeros(C)
     x_mean = zero if x_mean is None else x_mean
     t_mean = zero if t_mean is None else t_mean
     x_std = one if x_std is None else x_std
     t_std = one if t_std is None else t_std
     t_steps = sigma_schedule(n_diffusion, sigma_min, sigma_max, sigma_data)
+
+    def bcast(t):
+        return t.expand(B, *t.shape[1:])
+
     cond = state0.clone()
     X_un = state0 * x_std + x_mean
     states = []
-    for _ in range(n_forecast):
-        c = cond if extra_cond is None else torch.cat([cond, extra_cond], dim=2)
-        lat = torch.randn(state0.shape, generator=generator)
+    for k in range(n_forecast):
+        parts = [cond]
+        if forcing is not None:
+            parts.append(bcast(forcing[k]))
+        if static is not None:
+            parts.append(bcast(static))
+        if forcing is not None:
+            parts.append(bcast(forcing[k + 1]))
+        if extra_cond is not None:
+            parts.append(bcast(extra_cond if extra_cond.dim() == 3 else extra_cond[k]))
+        c = torch.cat(parts, dim=2)
+        lat = latents[k] if latents is not None else torch.randn(state0.shape, generator=generator)
         y = sample(denoiser, c, lat, t_steps, sigma_data)
         X_un = X_un + (y * t_std + t_mean)
         cond = (X_un - x_mean) / x_std

@@ -374,14 +374,21 @@ def output_stage(cfg: OracleConfig, sd, x, t_emb):
     return modulate(y, shift, scale) @ sd["output_stage.head.weight"].T
 
 
-def model_forward(cfg: OracleConfig, sd, x, dt, ape=None, return_hidden=False):
-    """Full denoiser forward (model.py:468-477): odd Swin layers run on the half-window-rolled grid."""
+def model_forward(cfg: OracleConfig, sd, x, dt, ape=None, return_hidden=False, block_hook=None):
+    """Full denoiser forward (model.py:468-477): odd Swin layers run on the half-window-rolled grid.
+    ``block_hook(k, hidden)`` sees the residual stream after the embedding (k = 0) and after block k."""
     tok, t_emb = input_stage(cfg, sd, x, dt, ape)
     wy, wx = cfg.window_size
+    k = 0
+    if block_hook is not None:
+        block_hook(0, tok)
     for i in range(cfg.n_layers - 2):
         shift = (wy // 2, wx // 2) if i % 2 == 1 else (0, 0)
         for j in range(cfg.sublayers):
             tok = block_forward(cfg, sd, tok, t_emb, shift, prefix=f"layers.{i}.modulelist.{j}.")
+            k += 1
+            if block_hook is not None:
+                block_hook(k, tok)
     out = output_stage(cfg, sd, tok, t_emb)
     if return_hidden:
         return out, tok

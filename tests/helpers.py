@@ -14,6 +14,10 @@ def rel_l2(a, b):
     return float((a - b).norm() / b.norm().clamp_min(1e-30))
 
 
+def max_abs(a, b):
+    return float((a.double().cpu() - b.double().cpu()).abs().max())
+
+
 def block_options(cfg: OracleConfig):
     return {k: getattr(cfg, k) for k in BLOCK_FIELDS}
 

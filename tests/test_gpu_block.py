@@ -11,7 +11,7 @@ import torch
 
 import oracle
 from oracle import OracleConfig
-from helpers import make_layer, make_model, rel_l2
+from helpers import make_layer, make_model, rel_l2, max_abs
 
 pytestmark = pytest.mark.gpu
 
@@ -159,10 +159,54 @@ def test_sampler_parity_and_graph_replay(pkg, cuda):
         replay = smp.sample_graph(c2, l2).clone()
         torch.cuda.synchronize()
         assert torch.equal(eager, replay), k
-    # autoregressive rollout against the oracle's
-    states = smp.rollout(cond[..., :8].contiguous().to(cuda), 2, torch.Generator(device="cuda").manual_seed(3),
-                         extra_cond=cond[..., 8:].contiguous().to(cuda))
-    assert len(states) == 2 and all(torch.isfinite(s).all() for s in states)
+
+
+def test_rollout_parity_eager_and_graph(pkg, cuda):
+    """Autoregressive rollout (inference.py:127-186) against the oracle's on the same latents: per-step forcings
+    (cat([state, rad_T[k], gp, lsm, rad_T[k+1]]), inference.py:133), non-identity per-channel means / stds for the
+    un-standardise / accumulate / re-standardise feedback (era5.py:95-114), two ensemble members as batch; eagerly and
+    with the whole forecast step replayed as one HIP graph (bit-identical to eager, also on later replays with eager
+    work in between)."""
+    C, Cf, Cs, n_fc, n_diff = 8, 3, 2, 3, 3
+    cfg = OracleConfig.ref(n_layers=4, in_channels=2 * C + 2 * Cf + Cs, out_channels=C, dim=128, heads=2, head_dim=64,
+                           mlp_dim=256, window_size=(8, 8), image_shape=(16, 24))
+    sd = oracle.init_model_weights(cfg, 6, nontrivial=True)
+    model = make_model(pkg, cfg, sd, cuda, torch.float32, "ref")
+    g = torch.Generator().manual_seed(12)
+    B, S = 2, 16 * 24
+    state0 = torch.randn(B, S, C, generator=g)
+    forcing = torch.randn(n_fc + 1, 1, S, Cf, generator=g)
+    static = torch.randn(1, S, Cs, generator=g)
+    lat = torch.randn(n_fc, B, S, C, generator=g)
+    x_mean, x_std = torch.randn(C, generator=g), 0.5 + torch.rand(C, generator=g)
+    t_mean, t_std = 0.1 * torch.randn(C, generator=g), 0.2 + 0.2 * torch.rand(C, generator=g)
+    kw = dict(x_mean=x_mean, x_std=x_std, t_mean=t_mean, t_std=t_std, forcing=forcing, static=static, latents=lat)
+    want = oracle.rollout(lambda m, t: oracle.model_forward(cfg, sd, m, t), state0, n_fc, n_diff, **kw)
+    smp = pkg.TrigFlowSampler(model, n_steps=n_diff, device=cuda)
+    dkw = {k: v.to(cuda) for k, v in kw.items()}
+    eager = smp.rollout(state0.to(cuda), n_fc, **dkw).clone()
+    torch.cuda.synchronize()
+    assert eager.shape == (n_fc, B, S, C)
+    for k in range(n_fc):
+        err = rel_l2(eager[k], want[k])
+        print(f"rollout step {k}: rel-L2 {err:.3e}, max-abs {max_abs(eager[k], want[k]):.3e}")
+        assert err <= 1e-2, (k, err)
+    assert rel_l2(eager[1], eager[0]) > 5e-2  # the steps differ: the feedback and the per-step forcings are live
+    ro = smp.begin_rollout(state0.to(cuda), n_fc, use_graph=True, graph_warmup=1, **dkw)
+    graph = ro.run().clone()
+    torch.cuda.synchronize()
+    assert torch.equal(graph, eager)
+    ro.reset()
+    for k in range(n_fc):  # replays with eager kernels and a synchronisation in between
+        ro.run(1)
+        model(torch.randn(B, S, cfg.in_channels, device=cuda), torch.tensor([0.3], device=cuda))
+        torch.cuda.synchronize()
+        assert torch.equal(ro.states[k], eager[k]), k
+    # a generator instead of given latents: the graph draws its latents on the device, every replay new ones
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    drawn = smp.rollout(state0.to(cuda), 2, gen, use_graph=True, **{k: v for k, v in dkw.items() if k != "latents"})
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(drawn).all()) and rel_l2(drawn[1], drawn[0]) > 5e-2
 
 
 @pytest.mark.parametrize("name,geo", [("config2", dict(dim=1024, heads=16, head_dim=64, mlp_dim=4096)),

@@ -1,0 +1,90 @@
+"""Parity at the depth and width the headline number is quoted on: 24 blocks, dim 1536, against the fp32 CPU oracle.
+
+The grid is the only thing that is reduced (the oracle has to finish in seconds): every kernel sees the row
+length, head count, window size and weight shapes of the benchmarked step, and the residual stream passes
+through all 24 blocks.  After every block the hidden state is compared (relative L2 and max-abs), which gives the
+error-growth curve; the final output has to be within the benchmark's tolerance of 1e-2 relative L2.
+The curves are printed and, where the directory can be written, stored as JSON under gpurun_out/.
+"""
+import json
+import os
+
+import pytest
+import torch
+
+import oracle
+from oracle import OracleConfig
+from helpers import make_model, rel_l2, max_abs
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def depth_curve(pkg, cuda, cfg, preset, res_dt, seed, grid_tokens, dt_value=0.9, use_ape=False):
+    sd = oracle.init_model_weights(cfg, seed)  # the benchmark's init: trunc-normal(0.02) matrices, zero biases, unit gains
+    model = make_model(pkg, cfg, sd, cuda, res_dt, preset)
+    g = torch.Generator().manual_seed(seed + 1)
+    x, dt = torch.randn(1, grid_tokens, cfg.in_channels, generator=g), torch.tensor([dt_value])
+    ape = None
+    if use_ape:
+        H, W = cfg.image_shape
+        ape = oracle.positional_encoding_2d(cfg.in_channels, H + 1, W)[1:].reshape(1, H * W, cfg.in_channels)
+        model.generate_ape()
+    want_h, got_h = [], []
+    with torch.no_grad():
+        want = oracle.model_forward(cfg, sd, x, dt, ape=ape, block_hook=lambda k, h: want_h.append(h.clone()))
+        got = model(x.to(cuda), dt.to(cuda), block_hook=lambda k, h: got_h.append(h.float().cpu()))
+        torch.cuda.synchronize()
+    assert len(want_h) == len(got_h) == (cfg.n_layers - 2) * cfg.sublayers + 1
+    curve = [{"block": k, "rel_l2": rel_l2(b, a), "max_abs": max_abs(b, a), "ref_rms": float(a.double().pow(2).mean().sqrt())}
+             for k, (a, b) in enumerate(zip(want_h, got_h))]
+    final = {"rel_l2": rel_l2(got, want), "max_abs": max_abs(got, want), "ref_rms": float(want.double().pow(2).mean().sqrt())}
+    return curve, final
+
+
+def report(tag, curve, final, extra):
+    print(f"\n[{tag}] hidden state after block k vs fp32 oracle: k, rel-L2, max-abs, rms of the oracle's")
+    for c in curve:
+        print(f"[{tag}] {c['block']:2d}  {c['rel_l2']:.3e}  {c['max_abs']:.3e}  {c['ref_rms']:.3f}")
+    print(f"[{tag}] output: rel-L2 {final['rel_l2']:.3e}, max-abs {final['max_abs']:.3e}, rms {final['ref_rms']:.3e}", flush=True)
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, f"depth_parity_{tag}.json"), "w") as f:
+            json.dump({"tag": tag, **extra, "hidden": curve, "output": final}, f, indent=1)
+    except OSError:
+        pass
+
+
+@pytest.mark.parametrize("res_dt", [torch.bfloat16, torch.float32], ids=["bf16_residual", "f32_residual"])
+def test_config3_depth_24_blocks(pkg, cuda, res_dt):
+    """configs[3]'s denoiser (138 -> dim 1536 -> 24 blocks of 24 x 64 heads, 16x16 windows alternately un-shifted and
+    shifted by 8 with mask and rel-pos bias, LayerNorm + scale/shift modulation, GELU MLP 6144 -> 69) on a 64x128 grid."""
+    H, W = 64, 128
+    cfg = OracleConfig.spec(n_layers=26, in_channels=138, out_channels=69, dim=1536, heads=24, head_dim=64, mlp_dim=6144,
+                            window_size=(16, 16), image_shape=(H, W), mod_ways=2)
+    curve, final = depth_curve(pkg, cuda, cfg, "spec", res_dt, 3, H * W)
+    tag = "config3_" + ("bf16" if res_dt == torch.bfloat16 else "f32") + "_residual"
+    report(tag, curve, final, {"grid": [H, W], "preset": "spec, mod_ways 2", "blocks": 24, "dim": 1536})
+    if res_dt == torch.float32:  # the default residual stream of LocalAERIS: inside the tolerance at every depth
+        assert final["rel_l2"] <= 1e-2, final
+        assert max(c["rel_l2"] for c in curve) <= 1e-2, curve
+    else:
+        # A bf16 residual stream (what the reference's bf16 layers keep) rounds the stream twice per block; after 24
+        # blocks that alone is about 1e-2 of the stream, and the output leaves the tolerance (measured 1.2e-2).  It is
+        # inside up to about 15 blocks.  This case records the curve and bounds it; it is why f32 is the default.
+        assert max(c["rel_l2"] for c in curve[:13]) <= 1e-2, curve
+        assert final["rel_l2"] <= 2e-2, final
+
+
+def test_reference_block_depth_24_blocks(pkg, cuda):
+    """The reference's own model shape (model.py:358-403, train.yaml: dim 1536, 12 heads x 128, SwiGLU 6144, 60x60 windows,
+    8 layers x 3 sublayers = 24 blocks, RMSNorm, 6-way modulation before the norm, APE on the inputs) on a 120x120 grid."""
+    H, W = 120, 120
+    cfg = OracleConfig.ref(n_layers=10, sublayers=3, in_channels=144, out_channels=70, dim=1536, heads=12, head_dim=128,
+                           mlp_dim=6144, window_size=(60, 60), image_shape=(H, W))
+    curve, final = depth_curve(pkg, cuda, cfg, "ref", torch.float32, 5, H * W, use_ape=True)
+    report("refwin_f32_residual", curve, final, {"grid": [H, W], "preset": "ref", "blocks": 24, "dim": 1536})
+    assert final["rel_l2"] <= 1e-2, final
+    assert max(c["rel_l2"] for c in curve) <= 1e-2, curve

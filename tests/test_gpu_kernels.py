@@ -92,9 +92,11 @@ def test_gemm_parity(pkg, cuda, case):
 def test_gemm_gelu_epilogue_pointwise(pkg, cuda):
     """The GELU of the GEMM epilogue, value by value: with one non-zero column in A and ones in W every output is
     GELU(x) for a chosen x.  Against the erf form in float64: the epilogue's polynomial is within 2.1e-4 |x| (a tenth of
-    half a bf16 ulp; beyond |x| = 3.5 this is the clamp's 1 - Phi(3.5)) before the result is rounded to bf16."""
+    half a bf16 ulp; above 3.5 this is the clamp's 1 - Phi(3.5)) before the result is rounded to bf16; below -3.5,
+    however far, it is the constant -8.1e-4 (the exact value lies between that and 0)."""
     M, N, K = 8192, 256, 64
-    x = bf(torch.cat([torch.linspace(-8, 8, M - 2048), torch.linspace(-0.05, 0.05, 2048)]))
+    x = bf(torch.cat([torch.linspace(-8, 8, M - 2048 - 512), torch.linspace(-0.05, 0.05, 2048),
+                      -torch.logspace(math.log10(3.5), 4, 256), torch.logspace(math.log10(3.5), 4, 256)]))
     a = torch.zeros(M, K, dtype=torch.bfloat16)
     a[:, 0] = x
     w = torch.zeros(N, K, dtype=torch.bfloat16)
@@ -102,7 +104,7 @@ def test_gemm_gelu_epilogue_pointwise(pkg, cuda):
     out = pkg.ops.gemm(a.to(cuda), w.to(cuda), None, act="gelu").float().cpu()
     xd = x.double()
     exact = 0.5 * xd * (1.0 + torch.erf(xd / math.sqrt(2.0)))
-    bound = 2.1e-4 * xd.abs() + 2.0 ** -8 * exact.abs() + 1e-30
+    bound = torch.where(xd >= -3.5, 2.1e-4 * xd.abs(), torch.full_like(xd, 8.2e-4)) + 2.0 ** -8 * exact.abs() + 1e-30
     err = (out.double() - exact[:, None]).abs()
     assert bool((err <= bound[:, None]).all()), float((err / bound[:, None]).max())
     assert torch.equal(out, out[:, :1].expand_as(out))  # every column took the same path
@@ -393,6 +395,24 @@ def test_embed_prepare_parity(pkg, cuda):
     out = pkg.ops.embed_prepare(x.to(cuda), None, 192).cpu()
     ref[:, :C] = x
     assert torch.equal(out, ref.to(torch.bfloat16))
+
+
+def test_embed_prepare_split_layout(pkg, cuda):
+    """split: every value v is written as [hi | lo | hi | 1 | 1], hi = bf16(v), lo = bf16(v - hi), zero padded: hi + lo
+    reproduces v to 2^-16 relative, and the concatenating form writes the same."""
+    g = torch.Generator().manual_seed(4)
+    M, C, K = 500, 138, 448
+    x, ape = torch.randn(M, C, generator=g) * 3, torch.randn(100, C, generator=g)
+    out = pkg.ops.embed_prepare(x.to(cuda), ape.to(cuda), K, split=True).cpu()
+    v = x + ape.repeat(5, 1)
+    hi = v.to(torch.bfloat16)
+    lo = (v - hi.float()).to(torch.bfloat16)
+    assert torch.equal(out[:, :C], hi) and torch.equal(out[:, C:2 * C], lo) and torch.equal(out[:, 2 * C:3 * C], hi)
+    assert torch.equal(out[:, 3 * C:3 * C + 2].float(), torch.ones(M, 2)) and not out[:, 3 * C + 2:].any()
+    assert float(((hi.float() + lo.float()) - v).abs().max() / v.abs().max()) < 2.0 ** -15
+    got = pkg.ops.embed_concat(x[:, :69].contiguous().to(cuda), 1.0, x[:, 69:].contiguous().to(cuda), ape.to(cuda), K,
+                               split=True).cpu()
+    assert torch.equal(got, out)
 
 
 def test_embed_concat_equals_cat_then_prepare(pkg, cuda):

@@ -117,10 +117,12 @@ def test_argument_validation_needs_no_gpu(pkg):
     # small ops
     assert lib.aeris_modulation_linear_fwd(p16, p16, None, p16, 1, 8, 12, 0, 0, None) == L.EUNSUPPORTED
     assert lib.aeris_timestep_embedding_fwd(p16, p16, 1, 7, 10000.0, None) == L.EINVAL
-    assert lib.aeris_embed_prepare_fwd(p16, None, p16, 4, 0, 138, 128, None) == L.EINVAL  # K_pad < C
-    assert lib.aeris_embed_concat_fwd(p16, 69, 1.0, p16, 69, None, p16, 4, 0, 128, None) == L.EINVAL  # K_pad < C0 + C1
-    assert lib.aeris_embed_concat_fwd(p16, 69, 0.0, p16, 69, None, p16, 4, 0, 192, None) == L.EINVAL  # div0 == 0
-    assert lib.aeris_embed_concat_fwd(p16, 69, 1.0, None, 69, None, p16, 4, 0, 192, None) == L.EINVAL  # x1 NULL
+    assert lib.aeris_embed_prepare_fwd(p16, None, p16, 4, 0, 138, 128, 0, None) == L.EINVAL  # K_pad < C
+    assert lib.aeris_embed_prepare_fwd(p16, None, p16, 4, 0, 138, 384, 1, None) == L.EINVAL  # split: K_pad < 3 C + 2
+    assert lib.aeris_embed_concat_fwd(p16, 69, 1.0, p16, 69, None, p16, 4, 0, 128, 0, None) == L.EINVAL  # K_pad < C0 + C1
+    assert lib.aeris_embed_concat_fwd(p16, 69, 1.0, p16, 69, None, p16, 4, 0, 384, 1, None) == L.EINVAL  # split: too narrow
+    assert lib.aeris_embed_concat_fwd(p16, 69, 0.0, p16, 69, None, p16, 4, 0, 192, 0, None) == L.EINVAL  # div0 == 0
+    assert lib.aeris_embed_concat_fwd(p16, 69, 1.0, None, 69, None, p16, 4, 0, 192, 0, None) == L.EINVAL  # x1 NULL
     with pytest.raises(pkg.AerisError):
         L.call("aeris_window_index_map", 1, 10, 8, 4, 4, 0, 0, p)
 

@@ -300,3 +300,47 @@ def test_rollout_feedback():
         y = torch.randn(state0.shape, generator=g2)
         X = X + (y * tsd + tm)
         torch.testing.assert_close(states[k], (X - xm) / xs)
+
+
+def test_rollout_conditioning_order_and_step_indexing():
+    """Known answer for the per-step conditioning of inference.py:133, cat([state, rad_T[k], gp, lsm, rad_T[k+1]]): a
+    probe denoiser that returns one input channel makes F constant in x, so the sampler's result is
+    x_N = sigma_d * (latents + (t_N - t_0) * F) = sigma_d * (latents - t_0 * F) whatever the number of Heun steps;
+    reading a different channel per probe shows which tensor (and which forecast step's slice) sits where."""
+    B, S, C, Cf, Cs, Ce, n_fc, n_diff, sd_ = 2, 5, 3, 2, 2, 1, 3, 4, 1.5
+    g = torch.Generator().manual_seed(2)
+    state0 = torch.randn(B, S, C, generator=g, dtype=torch.float64)
+    forcing = torch.randn(n_fc + 1, 1, S, Cf, generator=g, dtype=torch.float64)  # one batch entry: broadcast over members
+    static = torch.randn(B, S, Cs, generator=g, dtype=torch.float64)
+    extra = torch.randn(n_fc, B, S, Ce, generator=g, dtype=torch.float64)
+    lat = torch.randn(n_fc, B, S, C, generator=g, dtype=torch.float64)
+    t0 = oracle.sigma_schedule(n_diff, sigma_data=sd_)[0].double()
+    # channel layout the denoiser sees: [x / sigma_d (C) | state (C) | forcing[k] (Cf) | static (Cs) | forcing[k+1] (Cf) | extra[k] (Ce)]
+    off_state, off_f0, off_st, off_f1, off_ex = C, 2 * C, 2 * C + Cf, 2 * C + Cf + Cs, 2 * C + 2 * Cf + Cs
+    probes = {
+        "forcing[k]": (off_f0 + 1, lambda k: forcing[k, :, :, 1].expand(B, S)),
+        "static": (off_st, lambda k: static[:, :, 0]),
+        "forcing[k+1]": (off_f1, lambda k: forcing[k + 1, :, :, 0].expand(B, S)),
+        "extra[k]": (off_ex, lambda k: extra[k, :, :, 0]),
+    }
+    for name, (ch, want_fn) in probes.items():
+        seen_width = []
+
+        def den(m, t, ch=ch):
+            seen_width.append(m.shape[-1])
+            return m[..., ch:ch + 1].expand(-1, -1, C)
+
+        states = oracle.rollout(den, state0, n_fc, n_diff, sigma_data=sd_, forcing=forcing, static=static, extra_cond=extra,
+                                latents=lat)
+        assert set(seen_width) == {2 * C + 2 * Cf + Cs + Ce}
+        X = state0.clone()
+        for k in range(n_fc):
+            X = X + sd_ * (lat[k] - t0 * want_fn(k).unsqueeze(-1))
+            torch.testing.assert_close(states[k], X, rtol=1e-5, atol=1e-5, msg=name)
+    # the state itself is the first conditioning block, and it is the fed-back one from the second step on
+    states = oracle.rollout(lambda m, t: m[..., off_state:off_state + C], state0, 2, n_diff, sigma_data=sd_, forcing=forcing,
+                            static=static, latents=lat[:2])
+    X1 = state0 + sd_ * (lat[0] - t0 * state0)
+    X2 = X1 + sd_ * (lat[1] - t0 * X1)
+    torch.testing.assert_close(states[0], X1, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(states[1], X2, rtol=1e-5, atol=1e-5)

@@ -199,6 +199,56 @@ int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, co
   return AERIS_OK;
 }
 
+int64_t aeris_output_stage_workspace_bytes(int N, int d, int B_mod) {
+  if (B_mod <= 0 || !aeris::output_stage_supported(N, d)) return 0;
+  return aeris::output_stage_workspace_bytes(N, d, B_mod);
+}
+
+namespace {
+// shared argument checks of the output-stage entry points; sets *B_mod to the number of modulation rows in use
+int check_output_stage(const char* who, const void* x, int x_dtype, const void* gamma, const void* beta, int param_dtype,
+                       const float* shift, const float* scale, int64_t mod_batch_stride, const float* head_w, float* out,
+                       int64_t B, int64_t rows_per_batch, int N, int d, int kind, float eps, int* B_mod) {
+  if (!x || !gamma || !head_w || !out) return fail(AERIS_EINVAL, "%s: x/gamma/head_w/out is NULL", who);
+  if (!aligned16(x) || !aligned16(out) || !aligned16(head_w)) return fail(AERIS_EINVAL, "%s: x/out/head_w must be 16-byte aligned", who);
+  if (B <= 0 || rows_per_batch <= 0) return fail(AERIS_EINVAL, "%s: B and rows_per_batch must be positive", who);
+  if ((x_dtype != AERIS_BF16 && x_dtype != AERIS_F32) || (param_dtype != AERIS_BF16 && param_dtype != AERIS_F32))
+    return fail(AERIS_EINVAL, "%s: dtype must be AERIS_BF16 or AERIS_F32", who);
+  if (kind != AERIS_NORM_LAYER && kind != AERIS_NORM_RMS) return fail(AERIS_EINVAL, "%s: unknown norm kind %d", who, kind);
+  if (mod_batch_stride < 0) return fail(AERIS_EINVAL, "%s: negative mod_batch_stride", who);
+  if (!(eps >= 0.f)) return fail(AERIS_EINVAL, "%s: eps must be non-negative", who);
+  if (N <= 0 || d <= 0) return fail(AERIS_EINVAL, "%s: N and d must be positive", who);
+  if (!aeris::output_stage_supported(N, d))
+    return fail(AERIS_EUNSUPPORTED, "%s: N=%d, d=%d (need N <= 80 and d a multiple of 64)", who, N, d);
+  const bool batched = (shift || scale) && mod_batch_stride != 0 && B > 1;
+  if (batched && rows_per_batch % 64)
+    return fail(AERIS_EUNSUPPORTED, "%s: with one modulation row per batch entry rows_per_batch=%lld must be a multiple of 64",
+                who, (long long)rows_per_batch);
+  if (batched && B > 0x7fffffffLL / 1024) return fail(AERIS_EUNSUPPORTED, "%s: too many batch entries", who);
+  if ((B * rows_per_batch + 63) / 64 > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "%s: too many rows", who);
+  *B_mod = batched ? (int)B : 1;
+  return AERIS_OK;
+}
+}  // namespace
+
+int aeris_output_stage_fwd(const void* x, int x_dtype, const void* gamma, const void* beta, int param_dtype,
+                           const float* shift, const float* scale, int64_t mod_batch_stride, const float* head_w, float* out,
+                           int64_t B, int64_t rows_per_batch, int N, int d, int kind, float eps, void* workspace,
+                           int64_t workspace_bytes, void* stream) {
+  int B_mod = 1;
+  if (int rc = check_output_stage("aeris_output_stage_fwd", x, x_dtype, gamma, beta, param_dtype, shift, scale,
+                                  mod_batch_stride, head_w, out, B, rows_per_batch, N, d, kind, eps, &B_mod))
+    return rc;
+  const int64_t need = aeris::output_stage_workspace_bytes(N, d, B_mod);
+  if (!workspace || !aligned16(workspace) || workspace_bytes < need)
+    return fail(AERIS_EINVAL, "aeris_output_stage_fwd: workspace must be 16-byte aligned and hold %lld bytes (got %lld)",
+                (long long)need, (long long)workspace_bytes);
+  hipError_t e = aeris::output_stage_launch(x, x_dtype, gamma, beta, param_dtype, shift, scale, mod_batch_stride, head_w, out,
+                                            B, rows_per_batch, N, d, kind, eps, workspace, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_output_stage_fwd launch");
+  return AERIS_OK;
+}
+
 int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, const float* gate, const void* residual,
                    int64_t M, int N, int K, int64_t ldc, int act, int res_dtype, int c_dtype,
                    int64_t gate_batch_stride, int64_t rows_per_batch, void* stream) {

@@ -33,6 +33,14 @@ hipError_t norm_modulate_launch(const void* x, int x_dtype, void* y, int y_dtype
                                 int param_dtype, const float* shift, const float* scale, int64_t mod_batch_stride, int64_t B,
                                 int64_t rows_per_batch, int d, int kind, int order, float eps, hipStream_t stream);
 
+// fused output stage (output_stage.hip): norm -> modulate -> head in one pass; N <= 80, d % 64 == 0
+bool output_stage_supported(int N, int d);
+int64_t output_stage_workspace_bytes(int N, int d, int B_mod);
+hipError_t output_stage_launch(const void* x, int x_dtype, const void* gamma, const void* beta, int param_dtype,
+                               const float* shift, const float* scale, int64_t mod_batch_stride, const float* head_w,
+                               float* out, int64_t B, int64_t rows_per_batch, int N, int d, int kind, float eps,
+                               void* workspace, hipStream_t stream);
+
 hipError_t modulation_linear_launch(const float* x, const void* W, const void* bias, float* y, int B, int N, int K,
                                     int w_dtype, int act, hipStream_t stream);
 hipError_t timestep_embedding_launch(const float* t, float* emb, int B, int dim, float max_period, hipStream_t stream);

@@ -379,7 +379,9 @@ class InputStage(nn.Module):
 
 
 class OutputStage(nn.Module):
-    """norm -> modulate(shift, scale) -> head  (model.py:405-429); f32 parameters and f32 output."""
+    """norm -> modulate(shift, scale) -> head  (model.py:405-429); f32 parameters, f32 arithmetic accuracy and f32
+    output like the reference's.  One fused kernel reads the tokens once (ops.output_stage); shapes it does not take
+    (more than 80 output channels, dim not a multiple of 64) run as norm kernel + bf16 GEMM."""
 
     def __init__(self, dim, model_out_channels, image_shape, data_dtype=torch.float32, *, norm="rmsnorm", eps=None):
         super().__init__()
@@ -404,8 +406,13 @@ class OutputStage(nn.Module):
         h = ops.modulation_linear(dt.float().contiguous(), l0.weight, l0.bias, silu=True)
         m = ops.modulation_linear(h, l2.weight, l2.bias)
         shift, scale = m.chunk(2, dim=1)  # model.py:425
-        y = ops.norm_modulate(x.contiguous(), self.norm.weight, getattr(self.norm, "bias", None), shift, scale,
-                              kind=self.norm_kind, order="norm_then_mod", eps=self.norm_eps)
+        beta = getattr(self.norm, "bias", None)
+        w = self.head.weight
+        if w.dtype == torch.float32 and ops.output_stage_supported(w.shape[0], d, m.shape[0] if b > 1 else 1, n):
+            return ops.output_stage(x.contiguous(), self.norm.weight, beta, shift, scale, w, kind=self.norm_kind,
+                                    eps=self.norm_eps)
+        y = ops.norm_modulate(x.contiguous(), self.norm.weight, beta, shift, scale, kind=self.norm_kind,
+                              order="norm_then_mod", eps=self.norm_eps)
         return ops.gemm(y, self._head_weight(), out_dtype=torch.float32).view(b, n, -1)
 
 

@@ -221,6 +221,46 @@ def norm_modulate(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Ten
     return out
 
 
+def output_stage_supported(N: int, d: int, B_mod: int, rows_per_batch: int) -> bool:
+    return L.lib().aeris_output_stage_workspace_bytes(N, d, max(B_mod, 1)) > 0 and (B_mod <= 1 or rows_per_batch % 64 == 0)
+
+
+def output_stage(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], shift: Optional[torch.Tensor],
+                 scale: Optional[torch.Tensor], head_w: torch.Tensor, *, kind: str = "rmsnorm", eps: float = 1e-5,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [B, S, d] (bf16 | f32) -> f32 [B, S, N] = head_w[N, d] applied to modulate(norm(x), shift, scale), one pass."""
+    _dev(x, "x")
+    if x.dim() != 3:
+        raise RuntimeError("x must be [B, S, d]")
+    B, S, d = x.shape
+    _dev(gamma, "gamma")
+    if gamma.dtype not in _DT or gamma.numel() != d:
+        raise RuntimeError("gamma must be bf16 or f32 [d]")
+    if beta is not None:
+        _dev(beta, "beta", gamma.dtype)
+    _dev(head_w, "head_w", torch.float32)
+    N = head_w.shape[0]
+    if head_w.shape[1] != d:
+        raise RuntimeError(f"head_w must be [N, {d}]")
+    sh_ptr, st1 = _rowvec(shift, "shift", d, B)
+    sc_ptr, st2 = _rowvec(scale, "scale", d, B)
+    if shift is not None and scale is not None and st1 != st2:
+        raise RuntimeError("shift and scale must share their batch stride")
+    stride = max(st1, st2)
+    b_mod = B if (stride and B > 1) else 1
+    need = L.lib().aeris_output_stage_workspace_bytes(N, d, b_mod)
+    ws = workspace("output_stage", (max(need, 16),), torch.uint8, x.device)
+    if out is None:
+        out = torch.empty(B, S, N, dtype=torch.float32, device=x.device)
+    else:
+        _dev(out, "out", torch.float32)
+    with _timed("output_stage", float(B * S * d * x.element_size() + B * S * N * 4), "byte"):
+        L.call("aeris_output_stage_fwd", x.data_ptr(), _DT[x.dtype], gamma.data_ptr(), _ptr(beta), _DT[gamma.dtype], sh_ptr,
+               sc_ptr, stride, head_w.data_ptr(), out.data_ptr(), B, S, N, d,
+               L.NORM_LAYER if kind == "layernorm" else L.NORM_RMS, float(eps), ws.data_ptr(), ws.numel(), _stream())
+    return out
+
+
 _ACT = {None: L.ACT_NONE, "none": L.ACT_NONE, "gelu": L.ACT_GELU, "swiglu": L.ACT_SWIGLU, "silu": L.ACT_SILU}
 
 

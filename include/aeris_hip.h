@@ -111,6 +111,23 @@ int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, co
                             int64_t B, int64_t rows_per_batch, int d, int kind, int order, float eps,
                             void* stream);
 
+/* Output stage in one pass: out f32 [B*rows_per_batch, N] = head_w * modulate(norm(x), shift, scale)
+ *   x [B*rows_per_batch, d] (x_dtype bf16|f32); gamma [d], beta [d] or NULL (param_dtype); shift, scale f32
+ *   [B_mod, d] or NULL (mod_batch_stride as for aeris_norm_modulate_fwd); head_w f32 [N, d] (nn.Linear layout, no bias)
+ *   kind: AERIS_NORM_LAYER | AERIS_NORM_RMS; the order is norm then modulate.
+ * Replaces x.to(float32) -> norm -> modulate -> head of OutputStage.forward (model.py:421-429) at its fp32 accuracy
+ * (bf16 MFMA on operands split into a bf16 head and remainder, fp32 accumulation) without writing the normalised
+ * tokens anywhere.  workspace: device memory of at least aeris_output_stage_workspace_bytes(N, d, B_mod) bytes, 16-byte
+ * aligned, borrowed for the call (the per-call fold of gamma, beta, shift, scale into the head weight lives there);
+ * B_mod = B when shift / scale carry one row per batch entry (mod_batch_stride != 0 and B > 1), otherwise 1.
+ * Supported: N <= 80, d % 64 == 0, and rows_per_batch % 64 == 0 when B_mod > 1; otherwise AERIS_EUNSUPPORTED (use
+ * aeris_norm_modulate_fwd + aeris_gemm_fwd). */
+int64_t aeris_output_stage_workspace_bytes(int N, int d, int B_mod);
+int aeris_output_stage_fwd(const void* x, int x_dtype, const void* gamma, const void* beta, int param_dtype,
+                           const float* shift, const float* scale, int64_t mod_batch_stride, const float* head_w,
+                           float* out, int64_t B, int64_t rows_per_batch, int N, int d, int kind, float eps,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+
 /* C[M,N] = epilogue(A[M,K] * W[N,K]^T).
  *   A bf16 [M,K] (lda = K); W bf16 [N,K] ([2N,K] for SWIGLU); bias bf16 [N] ([2N] for SWIGLU) or NULL
  *   epilogue: v = acc + bias; v = act(v); if gate: v *= gate[b, n]; if residual: v += residual[m, n]

@@ -74,7 +74,44 @@ def test_output_stage_alone(pkg, cuda, preset, x_dtype):
     e = rel_l2(out, want)
     print(f"output stage ({preset}, {x_dtype}): rel-L2 {e:.3e}, max-abs {max_abs(out, want):.3e}")
     assert out.dtype == torch.float32 and out.shape == (B, S, 69)
-    assert e <= 3e-3, e  # bf16 operands of the head GEMM
+    assert e <= 2e-5, e
+
+
+@pytest.mark.parametrize("case", [
+    # B, S, d, N, kind, x dtype, modulation rows, row mean
+    (1, 1000, 1536, 69, "layernorm", torch.float32, 1, 0.0),    # ragged row count (1000 = 15 tiles + 40 rows)
+    (3, 128, 1536, 70, "rmsnorm", torch.float32, 3, 0.0),       # one modulation row per batch entry
+    (2, 192, 256, 8, "layernorm", torch.bfloat16, 2, 0.0),      # one column fragment, bf16 tokens
+    (1, 4096, 1024, 80, "layernorm", torch.float32, 0, 0.0),    # no modulation at all, five full fragments
+    (1, 640, 1536, 69, "layernorm", torch.float32, 1, 100.0),   # rows with |mean| = 50 sigma: the provisional centre
+    (2, 100, 128, 33, "rmsnorm", torch.bfloat16, 1, 3.0),
+], ids=lambda c: f"B{c[0]}_S{c[1]}_d{c[2]}_N{c[3]}_{c[4]}_{'f32' if c[5] == torch.float32 else 'bf16'}_mod{c[6]}_mean{c[7]:g}")
+def test_output_stage_kernel_against_float64(pkg, cuda, case):
+    """aeris_output_stage_fwd against norm -> modulate -> Linear evaluated in float64 (torch.nn.functional)."""
+    B, S, d, N, kind, x_dt, mod_rows, mean = case
+    g = torch.Generator().manual_seed(B * 1000 + S + d + N)
+    x = (2.0 * torch.randn(B, S, d, generator=g) + mean * (1 + torch.rand(B, S, 1, generator=g))).to(x_dt)
+    gamma, beta = 1 + 0.2 * torch.randn(d, generator=g), 0.3 * torch.randn(d, generator=g)
+    w = torch.randn(N, d, generator=g) / d ** 0.5
+    m = 0.3 * torch.randn(max(mod_rows, 1), 2 * d, generator=g)
+    shift, scale = (m[:, :d], m[:, d:]) if mod_rows else (None, None)
+    xd = x.double()
+    if kind == "layernorm":
+        y = torch.nn.functional.layer_norm(xd, (d,), gamma.double(), beta.double(), 1e-5)
+    else:
+        y = torch.nn.functional.rms_norm(xd, (d,), gamma.double(), 1e-6)
+    if mod_rows:
+        y = y * (1 + scale.double().unsqueeze(1)) + shift.double().unsqueeze(1)
+    want = y @ w.double().T
+    dev = lambda t: None if t is None else t.to(cuda)
+    md = m.to(cuda)
+    out = pkg.ops.output_stage(dev(x), dev(gamma), dev(beta) if kind == "layernorm" else None,
+                               md[:, :d] if mod_rows else None, md[:, d:] if mod_rows else None, dev(w), kind=kind,
+                               eps=1e-5 if kind == "layernorm" else 1e-6)
+    torch.cuda.synchronize()
+    e = rel_l2(out, want)
+    print(f"fused output stage {case[:5]}: rel-L2 {e:.3e}, max-abs {max_abs(out, want):.3e}")
+    assert out.shape == (B, S, N) and e <= (2e-5 if mean < 50 else 2e-4), e
 
 
 def test_converted_checkpoint_runs_on_the_gpu(pkg, cuda, tmp_path):

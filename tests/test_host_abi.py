@@ -114,6 +114,21 @@ def test_argument_validation_needs_no_gpu(pkg):
     assert hh(p16, p16, p16, None, 8, 128, 64, 60, 8 * 60, None) == L.EINVAL  # head_dim % 8
     assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64 - 8, None) == L.EINVAL  # planes overlap
     assert hh(p16, None, p16, None, 8, 128, 64, 64, 8 * 64, None) == L.EINVAL  # W NULL
+    # fused output stage
+    osf, osw = lib.aeris_output_stage_fwd, lib.aeris_output_stage_workspace_bytes
+    assert osw(69, 1536, 1) == 1536 * 80 * 4 + 80 * 8 and osw(69, 1536, 4) == 4 * osw(69, 1536, 1)
+    assert osw(81, 1536, 1) == 0 and osw(69, 1500, 1) == 0 and osw(69, 1536, 0) == 0  # unsupported shapes: no size
+    ok = (p16, L.F32, p16, None, L.F32, None, None, 0, p16, p16, 1, 128, 69, 1536, L.NORM_RMS, 1e-6, p16, osw(69, 1536, 1), None)
+    def with_(i, v):
+        a = list(ok); a[i] = v; return a
+    assert osf(*with_(0, None)) == L.EINVAL and osf(*with_(8, None)) == L.EINVAL  # x / head_w NULL
+    assert osf(*with_(12, 81)) == L.EUNSUPPORTED and osf(*with_(13, 1500)) == L.EUNSUPPORTED
+    assert osf(*with_(17, osw(69, 1536, 1) - 1)) == L.EINVAL and "workspace" in L.last_error()
+    assert osf(*with_(16, None)) == L.EINVAL
+    assert osf(*with_(14, 7)) == L.EINVAL  # norm kind
+    # one modulation row per batch entry: rows_per_batch must be a multiple of the 64-row tile
+    a = list(ok); a[5] = p16; a[7] = 1536; a[10] = 2; a[11] = 100; a[17] = osw(69, 1536, 2)
+    assert osf(*a) == L.EUNSUPPORTED
     # small ops
     assert lib.aeris_modulation_linear_fwd(p16, p16, None, p16, 1, 8, 12, 0, 0, None) == L.EUNSUPPORTED
     assert lib.aeris_timestep_embedding_fwd(p16, p16, 1, 7, 10000.0, None) == L.EINVAL

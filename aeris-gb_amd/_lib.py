@@ -36,6 +36,8 @@ SIGNATURES = {
     "aeris_output_stage_workspace_bytes": (_c_i64, [_c_int, _c_int, _c_int]),
     "aeris_output_stage_fwd": (_c_int, [_c_vp, _c_int, _c_vp, _c_vp, _c_int, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_i64, _c_i64,
                                         _c_int, _c_int, _c_int, _c_f32, _c_vp, _c_i64, _c_vp]),
+    "aeris_output_stage_noalloc_fwd": (_c_int, [_c_vp, _c_int, _c_vp, _c_vp, _c_int, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_i64,
+                                                _c_i64, _c_int, _c_int, _c_int, _c_f32, _c_vp]),
     "aeris_gemm_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_i64, _c_int,
                                 _c_int, _c_int, _c_i64, _c_i64, _c_vp]),
     "aeris_gemm_heads_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_int, _c_i64, _c_vp]),

@@ -43,6 +43,14 @@ int ensure_init(void* stream = nullptr, bool from_launch = false) {
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_stream_configure_all();
     g_init_done.store(true, std::memory_order_release);
   });
+  if (g_init_status == hipSuccess && !from_launch) {
+    // aeris_init() itself: also resolve, for the device that is current now, the address of the scratch array
+    // that aeris_output_stage_noalloc_fwd uses (once per device; a later device gets it on its own aeris_init
+    // or on its first call of that entry point)
+    void* p = nullptr;
+    hipError_t e = aeris::output_stage_scratch(&p, true);
+    if (e != hipSuccess) return hip_fail(e, "aeris_init (hipGetSymbolAddress of the scratch array)");
+  }
   if (g_init_status != hipSuccess) return hip_fail(g_init_status, "aeris_init (hipFuncSetAttribute)");
   return AERIS_OK;
 }
@@ -246,6 +254,37 @@ int aeris_output_stage_fwd(const void* x, int x_dtype, const void* gamma, const 
   hipError_t e = aeris::output_stage_launch(x, x_dtype, gamma, beta, param_dtype, shift, scale, mod_batch_stride, head_w, out,
                                             B, rows_per_batch, N, d, kind, eps, workspace, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_output_stage_fwd launch");
+  return AERIS_OK;
+}
+
+int aeris_output_stage_noalloc_fwd(const void* x, int x_dtype, const void* gamma, const void* beta, int param_dtype,
+                                   const float* shift, const float* scale, int64_t mod_batch_stride, const float* head_w,
+                                   float* out, int64_t B, int64_t rows_per_batch, int N, int d, int kind, float eps,
+                                   void* stream) {
+  const char* who = "aeris_output_stage_noalloc_fwd";
+  int B_mod = 1;
+  if (int rc = check_output_stage(who, x, x_dtype, gamma, beta, param_dtype, shift, scale, mod_batch_stride, head_w, out, B,
+                                  rows_per_batch, N, d, kind, eps, &B_mod))
+    return rc;
+  const int64_t need = aeris::output_stage_workspace_bytes(N, d, B_mod), cap = aeris::output_stage_scratch_capacity();
+  if (need > cap)
+    return fail(AERIS_EUNSUPPORTED,
+                "%s: the fold of %d modulation row(s) at N=%d, d=%d needs %lld bytes, the library's scratch array holds "
+                "%lld: use aeris_output_stage_fwd with a workspace",
+                who, B_mod, N, d, (long long)need, (long long)cap);
+  // the array's address on this device: cached after the first look-up, which must not fall inside a capture
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  const bool capturing =
+      hipStreamIsCapturing(reinterpret_cast<hipStream_t>(stream), &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+  void* ws = nullptr;
+  hipError_t e = aeris::output_stage_scratch(&ws, !capturing);
+  if (e == hipErrorNotReady)
+    return fail(AERIS_EINVAL, "%s: first use on this device while the stream is being captured: call aeris_init() "
+                              "with this device current before the capture begins", who);
+  if (e != hipSuccess) return hip_fail(e, "aeris_output_stage_noalloc_fwd (scratch address)");
+  e = aeris::output_stage_launch(x, x_dtype, gamma, beta, param_dtype, shift, scale, mod_batch_stride, head_w, out, B,
+                                 rows_per_batch, N, d, kind, eps, ws, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_output_stage_noalloc_fwd launch");
   return AERIS_OK;
 }
 

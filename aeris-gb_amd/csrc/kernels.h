@@ -36,6 +36,10 @@ hipError_t norm_modulate_launch(const void* x, int x_dtype, void* y, int y_dtype
 // fused output stage (output_stage.hip): norm -> modulate -> head in one pass; N <= 80, d % 64 == 0
 bool output_stage_supported(int N, int d);
 int64_t output_stage_workspace_bytes(int N, int d, int B_mod);
+// the library's own scratch array for the entry point that allocates nothing: capacity in bytes, and its device
+// address on the current device (hipErrorNotReady when it has not been looked up yet and lookup_allowed is false)
+int64_t output_stage_scratch_capacity();
+hipError_t output_stage_scratch(void** ptr, bool lookup_allowed);
 hipError_t output_stage_launch(const void* x, int x_dtype, const void* gamma, const void* beta, int param_dtype,
                                const float* shift, const float* scale, int64_t mod_batch_stride, const float* head_w,
                                float* out, int64_t B, int64_t rows_per_batch, int N, int d, int kind, float eps,

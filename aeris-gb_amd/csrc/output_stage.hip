@@ -19,11 +19,22 @@
 // conflict-free ds_read_b128.
 #include "common.h"
 #include "kernels.h"
+#include <mutex>
 
 namespace aeris {
 
 namespace {
 constexpr int OS_ROWS = 64, OS_THREADS = 256;
+
+// Scratch of the entry point that allocates nothing (aeris_output_stage_noalloc_fwd): the per-call fold of the
+// modulation into the head weight lives in this array instead of a caller's workspace.  Every GPU the library runs
+// on holds its own copy until the process ends.  In host code the name below is only a handle: the array's device
+// address is looked up once per device with hipGetSymbolAddress and that pointer is what the kernels receive.
+constexpr int64_t OS_SCRATCH_BYTES = 2 << 20;
+static __device__ __align__(256) unsigned char scratch[OS_SCRATCH_BYTES];
+constexpr int OS_MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[OS_MAX_DEVICES] = {};
 
 struct OutStageParams {
   const void* x;
@@ -265,6 +276,27 @@ hipError_t launch_main(const OutStageParams& p, bool xf, bool ln, hipStream_t st
   return hipGetLastError();
 }
 }  // namespace
+
+int64_t output_stage_scratch_capacity() { return OS_SCRATCH_BYTES; }
+
+// Device address of `scratch` on the current device; looked up on the first call per device (hipGetSymbolAddress is
+// not a stream operation: make that first call, e.g. through aeris_init, outside any stream capture).
+hipError_t output_stage_scratch(void** ptr, bool lookup_allowed) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= OS_MAX_DEVICES) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    if (!lookup_allowed) return hipErrorNotReady;
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return hipSuccess;
+}
 
 bool output_stage_supported(int N, int d) { return N >= 1 && N <= 80 && d >= 64 && d % 64 == 0; }
 

@@ -128,6 +128,19 @@ int aeris_output_stage_fwd(const void* x, int x_dtype, const void* gamma, const 
                            float* out, int64_t B, int64_t rows_per_batch, int N, int d, int kind, float eps,
                            void* workspace, int64_t workspace_bytes, void* stream);
 
+/* aeris_output_stage_fwd without the workspace argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * per-call fold lives in an array of 2 MiB inside the library (one copy per GPU, held until the process ends); the
+ * call allocates and frees nothing.  Limit: aeris_output_stage_workspace_bytes(N, d, B_mod) <= 2 MiB (at N <= 80,
+ * d = 1536: up to 4 modulation rows), otherwise AERIS_EUNSUPPORTED.  Same kernels and results as
+ * aeris_output_stage_fwd.  Every call on a GPU uses that GPU's one array: calls that overlap in time on one GPU
+ * (two streams, two threads) race; order them on one stream.  The array's address is looked up on aeris_init() or
+ * on the first call per device, which must happen outside any stream capture. */
+int aeris_output_stage_noalloc_fwd(const void* x, int x_dtype, const void* gamma, const void* beta, int param_dtype,
+                                   const float* shift, const float* scale, int64_t mod_batch_stride,
+                                   const float* head_w, float* out, int64_t B, int64_t rows_per_batch, int N, int d,
+                                   int kind, float eps, void* stream);
+
 /* C[M,N] = epilogue(A[M,K] * W[N,K]^T).
  *   A bf16 [M,K] (lda = K); W bf16 [N,K] ([2N,K] for SWIGLU); bias bf16 [N] ([2N] for SWIGLU) or NULL
  *   epilogue: v = acc + bias; v = act(v); if gate: v *= gate[b, n]; if residual: v += residual[m, n]

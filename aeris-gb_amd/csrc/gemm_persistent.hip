@@ -42,11 +42,14 @@ constexpr int GM = 4;                     // row panels per L2 group
 // PLAIN: no gate and no residual (qkv, fc1): the epilogue is compiled without those paths - about 2 % faster than
 // deciding at run time, block by block, that there is nothing to load.  RES_BF16: bf16 C with a bf16 residual (proj,
 // fc2 on a bf16 residual stream), compiled as a kernel of its own so that its deeper residual prefetch does not
-// share registers with the general path.
-template <int ACT, bool OUT_F32, bool PLAIN, bool RES_BF16 = false>
+// share registers with the general path.  RES_F32: the same for f32 C with an f32 residual (proj, fc2 on an f32
+// residual stream).
+template <int ACT, bool OUT_F32, bool PLAIN, bool RES_BF16 = false, bool RES_F32 = false>
 __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams p_in) {
   static_assert(!(PLAIN && RES_BF16) && !(OUT_F32 && RES_BF16), "RES_BF16 is a non-plain bf16-output form");
+  static_assert(!RES_F32 || (OUT_F32 && !PLAIN && !RES_BF16), "RES_F32 is a non-plain f32-output form");
   GemmParams p = p_in;
+  if (RES_F32) p.res_dtype = AERIS_F32;
   if (PLAIN) {
     p.gate = nullptr;
     p.residual = nullptr;
@@ -488,6 +491,60 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           }
         }
       }
+    } else if (RES_F32 && ACT != AERIS_ACT_SWIGLU && rows_left == BM / WM && n_wave + BN / WN <= N && !gate_per_lane) {
+      // Interior tiles with f32 C and an f32 residual: the staging of the general f32 path below (units of 32 rows x
+      // 32 columns through the wave's 4 KB), as straight-line code without per-lane conditions, the residual rows
+      // requested two units ahead of their use and always ahead of the stores of the unit before.
+      constexpr int NU = FN / 2, UNITS = FM / 2 * NU;
+      const int n_lane = n_wave + rch * 4;
+      f32x4 gt[NU];
+#pragma unroll
+      for (int j = 0; j < NU; ++j) {
+        gt[j] = f32x4{1.f, 1.f, 1.f, 1.f};
+        if (gate_tile) gt[j] = *reinterpret_cast<const f32x4*>(gate_tile + n_lane + 32 * j);
+      }
+      const unsigned char* const res_lane = reinterpret_cast<const unsigned char*>(p.residual) + (m_base * p.ldc + n_lane) * 4;
+      unsigned char* const c_lane = reinterpret_cast<unsigned char*>(p.C) + (m_base * p.ldc + n_lane) * 4;
+      u32x4 rq[3][4];
+      auto load_res = [&](int u) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+          rq[u % 3][it] = *reinterpret_cast<const u32x4*>(
+              res_lane + ((int64_t)__mul24((u / NU) * 32 + rrow + 8 * it, ld24) + (u % NU) * 32) * 4);
+      };
+      load_res(0);
+#pragma unroll
+      for (int u = 0; u < UNITS; ++u) {
+        const int i = u / NU, j = u % NU;
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            float v[4];
+            fragment(2 * i + ii, 2 * j + jj, v);
+            *reinterpret_cast<f32x4*>(stg + swz_off(ii * 16 + l15, jj * 4 + q)) = f32x4{v[0], v[1], v[2], v[3]};
+          }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (u == 0) load_res(1);  // once the first unit's accumulators are staged and their registers free
+        f32x4 out[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          f32x4 o = *reinterpret_cast<const f32x4*>(stg + swz_off(rrow + 8 * it, rch));
+          o *= gt[j];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] += __uint_as_float(rq[u % 3][it][e]);
+          out[it] = o;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (u + 2 < UNITS) load_res(u + 2);  // ahead of the stores below
+        if (u + 1 == UNITS && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+          *reinterpret_cast<f32x4*>(c_lane + ((int64_t)__mul24(i * 32 + rrow + 8 * it, ld24) + j * 32) * 4) = out[it];
+      }
     } else {
       // stage 2 (f32 C): units of 32 rows x 32 columns (2 x 2 fragments), rows of 128 B (32 floats), 4 floats per
       // lane and row
@@ -673,6 +730,9 @@ hipError_t gemm_persistent_configure() {
   if (e != hipSuccess) return e;
   CFGR(AERIS_ACT_NONE) CFGR(AERIS_ACT_GELU) CFGR(AERIS_ACT_SWIGLU)
 #undef CFGR
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_persistent_kernel<AERIS_ACT_NONE, true, false, false, true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+  if (e != hipSuccess) return e;
   return hipSuccess;
 }
 
@@ -690,6 +750,10 @@ hipError_t gemm_persistent_launch(const GemmParams& p0, hipStream_t stream) {
   const bool f32 = p.c_dtype == AERIS_F32;
   const bool plain = !p.gate && p.res_dtype < 0;
   const bool res_bf16 = !f32 && p.res_dtype == AERIS_BF16;
+  if (f32 && p.res_dtype == AERIS_F32 && p.act == AERIS_ACT_NONE && !p.split) {
+    hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<AERIS_ACT_NONE, true, false, false, true>), grid, block, SMEM, stream, p);
+    return hipGetLastError();
+  }
 #define GO1(A, F32)                                                                                        \
   do {                                                                                                     \
     if (plain) hipLaunchKernelGGL((gemm_bf16_nt_persistent_kernel<A, F32, true>), grid, block, SMEM, stream, p);  \

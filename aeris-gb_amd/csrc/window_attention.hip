@@ -161,12 +161,11 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
         vreg[it][j] = *reinterpret_cast<const u32x4*>(vbase + (uint64_t)token_row(kg * 4 + j) * ld_qkv + c * 8);
     }
   }
-  const float inv_scale = 1.0f / p.scale;
   if (HAS_BIAS) {
 #pragma unroll
     for (int it = 0; it < BIT; ++it) {
       const int j = tid + it * NT;
-      breg[it] = j < TBL ? bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * inv_scale : 0.f;  // R[j]
+      breg[it] = j < TBL ? bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E : 0.f;  // R[j]
     }
   }
   // every load above is in flight before the first LDS write below waits for one of them
@@ -213,11 +212,25 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     }
     // tail components R4[s][e] with s+e >= TBL are never read by a valid key group
   }
+  // ---- q * scale * log2(e), rounded to bf16 once more: the accumulators of K Q^T are then the logits in the exp2
+  // domain and P = exp2(acc) needs no multiply
+  {
+    const float c = p.scale * LOG2E;
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps)
+#pragma unroll
+      for (int s2 = 0; s2 < KS; ++s2) {
+        u32x4 w = __builtin_bit_cast(u32x4, qf[ps][s2]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(bf16_lo(w[e]) * c, bf16_hi(w[e]) * c);
+        qf[ps][s2] = __builtin_bit_cast(bf16x8, w);
+      }
+  }
   __syncthreads();
 
   const bool my = p.use_mask && p.sy > 0 && wy == p.nWy - 1;
   const bool mx = p.use_mask && p.sx > 0 && wx == p.nWx - 1;
-  const float c = p.scale * LOG2E;
+  constexpr float MASK_NEG = -100.0f * LOG2E;  // the additive -100 of the shift mask, in the exp2 domain
 
 #pragma unroll
   for (int ps = 0; ps < 2; ++ps) {
@@ -226,16 +239,15 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     int qpos = qg * 32 + l31;
     const bool q_valid = qpos < L;
     if (!q_valid) qpos = L - 1;
-
-    // ---- S^T = K Q^T (+ bias / scale: the accumulators start at the relative-position bias, in the domain of the raw
-    // scores, so that logit * log2e = c * acc and the bias costs neither an add nor a zero-fill)
-    // The K fragments - and the bias vectors - of key block kb + 1 are read while the MFMAs of block kb run (left to
-    // itself the compiler reads each fragment right before its MFMA and exposes the LDS latency every time).
     const int qiy = qpos / WS_X, qix = qpos % WS_X;
     const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
-    f32x16 acc[NQ];
-    bf16x8 kf[2][KS];
-    auto init_acc = [&](int kb) {
+    const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
+    const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
+
+    // S^T block kb = K[32 kb ..] Q^T (+ bias): the accumulators start at the relative-position bias (read from LDS
+    // straight into them), so that it costs neither an add nor a zero-fill.
+    // a[4g+i] = logit * log2(e) of key 32 kb + 8 g + 4 hi + i and query qpos.
+    auto init_acc = [&](int kb, f32x16& a) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         f32x4 bv = {0.f, 0.f, 0.f, 0.f};
@@ -246,34 +258,17 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
           bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[kb][g * 4 + i] = bv[i];
+        for (int i = 0; i < 4; ++i) a[g * 4 + i] = bv[i];
       }
     };
+    auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) kf[0][s] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(l31, s * 2 + hi));
-    init_acc(0);
-#pragma unroll
-    for (int kb = 0; kb < NQ; ++kb) {
-      if (kb + 1 < NQ) {
-#pragma unroll
-        for (int s = 0; s < KS; ++s)
-          kf[(kb + 1) & 1][s] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>((kb + 1) * 32 + l31, s * 2 + hi));
-        init_acc(kb + 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int s = 0; s < KS; ++s) acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb & 1][s], qf[ps][s], acc[kb], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // acc[kb][4g+i] = <k[key], q[query]> + bias / scale, key = 32kb + 8g + 4hi + i, query = qpos
-
-    // ---- cyclic-shift mask: only windows touching the wrapped border carry more than one region
-    if (my || mx) {
-      const float neg = -100.0f / p.scale;  // becomes -100 after the scale multiply below
-      const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
-      const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb)
+      for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(kb * 32 + l31, s2 * 2 + hi));
+    };
+    // cyclic-shift mask (only windows touching the wrapped border carry more than one region) and the padding keys
+    // of windows whose token count is not a multiple of 32
+    auto mask_block = [&](int kb, f32x16& a) {
+      if (my || mx) {
 #pragma unroll
         for (int g = 0; g < 4; ++g)
 #pragma unroll
@@ -282,76 +277,146 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
             const int kiy = key / WS_X, kix = key % WS_X;
             const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
             const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
-            if (ry_k != ry_q || rx_k != rx_q) acc[kb][g * 4 + i] += neg;
+            if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
           }
-    }
-
-    // ---- row max of the logits (exp2 domain): the max of the raw scores is enough (scale > 0), the scale moves into
-    // the exp2 argument
-    float mrow = -INFINITY;
-#pragma unroll
-    for (int kb = 0; kb < NQ; ++kb)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const bool valid = (LPAD == L) || (kb * 32 + g * 8 + hi * 4) < L;
-        if (!valid) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[kb][g * 4 + i] = -INFINITY;
-        }
-        mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4]), acc[kb][g * 4 + 1]);
-        mrow = fmaxf(fmaxf(mrow, acc[kb][g * 4 + 2]), acc[kb][g * 4 + 3]);
       }
-    mrow *= c;
-    mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
-
-    // ---- P = exp2(t - max), row sum, pack to bf16 (the B operand of PV), and O^T = V^T P^T, 16 keys at a time.
-    // PV step (kb, t2): k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one
-    // V^T chunk per 32-row block of O^T.  While the MFMAs of a step run, the V^T fragments of the next step are read
-    // and its P is formed: the VALU work hides the MFMAs, and the LDS latency is a whole step away.
-    float sum = 0.f;
-    uint32_t pkb[2][4];
-    bf16x8 vfb[2][DB];
-    auto exp_step = [&](int step, uint32_t (&pk)[4]) {
-      const int kb = step >> 1, t2 = step & 1;
+      if (LPAD != L) {
 #pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const int h2 = 4 * t2 + h;
-        const float e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -mrow));
-        const float e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -mrow));
-        pk[h] = pack_bf16x2(e0, e1);
-        sum = dot2_ones(pk[h], sum);  // the row sum of what PV multiplies: the rounded values, one instruction per pair
+        for (int g = 0; g < 4; ++g)
+          if (kb * 32 + g * 8 + hi * 4 >= L) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[g * 4 + i] = -INFINITY;
+          }
       }
     };
+    // V^T fragment of PV step `step` (16 keys): k slots 0-3 <-> keys 16 step + 4hi + (0..3), slots 4-7 <-> keys
+    // 16 step + 8 + 4hi + (0..3): one 16-byte chunk per 32-row block of O^T
     auto load_v = [&](int step, bf16x8 (&f)[DB]) {
-      const int chunk = step * 2 + hi;  // 16-byte chunk of the row: 8 keys of this lane half
+      const int chunk = step * 2 + hi;
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const int d = db * 32 + l31;
         f[db] = *reinterpret_cast<const bf16x8*>(sV + d * VROW + ((chunk ^ v_swz<Cfg::V_SWZ>(d)) << 4));
       }
     };
+
     f32x16 o[DB];
+    float sum;
+
+    // ---- fast path: one sweep over the key blocks, P = exp2(logit) without subtracting the row maximum.
+    // softmax is invariant to the subtraction; it only guards the range, and the range is checked afterwards: a row
+    // sum outside [2^-40, 2^100] (or not finite) sends the wave to the two-pass form below.  Per key block the MFMAs
+    // of S^T for block kb + 1 are issued ahead of the exp2 of block kb, and those of P V for block kb after it: the
+    // matrix pipe runs while the VALU forms P.
+    {
+      f32x16 acc3[3];
+      bf16x8 kf[2][KS], vf[2][DB];
+      uint32_t pk[8];
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-    load_v(0, vfb[0]);
-    exp_step(0, pkb[0]);
-#pragma unroll
-    for (int step = 0; step < 2 * NQ; ++step) {
-      __builtin_amdgcn_sched_barrier(0);
-      if (step + 1 < 2 * NQ) {
-        load_v(step + 1, vfb[(step + 1) & 1]);
-        exp_step(step + 1, pkb[(step + 1) & 1]);
+        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+      sum = 0.f;
+      load_k(0, kf[0]);
+      init_acc(0, acc3[0]);
+      if (NQ > 1) {
+        load_k(1, kf[1]);
+        init_acc(1, acc3[1]);
       }
-      const uint32_t* pk = pkb[step & 1];
-      u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
-      const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfb[step & 1][db], pf, o[db], 0, 0, 0);
+      for (int s2 = 0; s2 < KS; ++s2)
+        acc3[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0][s2], qf[ps][s2], acc3[0], 0, 0, 0);
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb) {
+        f32x16& a = acc3[kb % 3];
+        __builtin_amdgcn_sched_barrier(0);
+        // LDS reads of this iteration: V^T fragments of the two PV steps of block kb; K fragments and bias of block kb + 2
+        load_v(2 * kb, vf[0]);
+        load_v(2 * kb + 1, vf[1]);
+        if (kb + 1 < NQ) {
+#pragma unroll
+          for (int s2 = 0; s2 < KS; ++s2)
+            acc3[(kb + 1) % 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[(kb + 1) & 1][s2], qf[ps][s2], acc3[(kb + 1) % 3], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (kb + 2 < NQ) {
+          load_k(kb + 2, kf[kb & 1]);
+          init_acc(kb + 2, acc3[(kb + 2) % 3]);
+        }
+        mask_block(kb, a);
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+          const float e0 = __builtin_amdgcn_exp2f(a[2 * h]);
+          const float e1 = __builtin_amdgcn_exp2f(a[2 * h + 1]);
+          pk[h] = pack_bf16x2(e0, e1);
+          sum = dot2_ones(pk[h], sum);  // the row sum of what PV multiplies: the rounded values
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          const u32x4 pw = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
+          const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+          for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t2][db], pf, o[db], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      sum += __shfl_xor(sum, 32, 64);
     }
-    __builtin_amdgcn_sched_barrier(0);
-    sum += __shfl_xor(sum, 32, 64);
+    const bool in_range = sum >= 0x1p-40f && sum <= 0x1p100f;  // false for NaN as well
+    if (__builtin_amdgcn_ballot_w64(!in_range) != 0) {
+      // ---- two-pass form for rows whose logits leave the range: all of S^T, row maximum, P = exp2(logit - max)
+      f32x16 acc[NQ];
+      bf16x8 kf[2][KS];
+      load_k(0, kf[0]);
+      init_acc(0, acc[0]);
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb) {
+        if (kb + 1 < NQ) {
+          load_k(kb + 1, kf[(kb + 1) & 1]);
+          init_acc(kb + 1, acc[kb + 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < KS; ++s2)
+          acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb & 1][s2], qf[ps][s2], acc[kb], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      float mrow = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb) {
+        mask_block(kb, acc[kb]);
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) mrow = fmaxf(fmaxf(mrow, acc[kb][e]), acc[kb][e + 1]);
+      }
+      mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
+      sum = 0.f;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+#pragma unroll
+      for (int step = 0; step < 2 * NQ; ++step) {
+        const int kb = step >> 1, t2 = step & 1;
+        bf16x8 vf[DB];
+        load_v(step, vf);
+        uint32_t pk[4];
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          const int h2 = 4 * t2 + h;
+          const float e0 = __builtin_amdgcn_exp2f(acc[kb][2 * h2] - mrow);
+          const float e1 = __builtin_amdgcn_exp2f(acc[kb][2 * h2 + 1] - mrow);
+          pk[h] = pack_bf16x2(e0, e1);
+          sum = dot2_ones(pk[h], sum);
+        }
+        const u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
+        const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf, o[db], 0, 0, 0);
+      }
+      sum += __shfl_xor(sum, 32, 64);
+    }
     const float inv = __builtin_amdgcn_rcpf(sum);
 
     // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i].  The two lanes of a query (l31 and

@@ -443,8 +443,759 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
 }
 
 // ---------------------------------------------------------------------------------------------
+// The same computation for head_dim 64 with K and V brought into LDS by the load unit itself
+// (buffer_load ... lds: no staging registers, no ds_write, no VALU work) and V kept row-major: the V^T fragments of
+// P V come from ds_read_b64_tr_b16, the LDS read that transposes on the way out.
+//   layout   K and V rows of 128 B, 16-byte chunks XOR-swizzled: K by (key >> 1) & 7 (16 consecutive keys of one chunk
+//            hit distinct banks for the ds_read_b128 fragments), V by 2 (key & 3) (the 4 keys x 4 column groups that
+//            one transposing read gathers per 16 lanes hit distinct banks).  A load instruction of a wave fills 1 KB =
+//            8 rows; lane l fetches the chunk that the swizzle keeps at its LDS slot, from the folded token row.
+//   tr read  within 16 lanes, source lane 4e + a reads 4 consecutive elements and result lane 4a + b receives element b
+//            of the source lanes a, 4 + a, 8 + a, 12 + a: with source lane 4e + a at V[key0 + e][d0 + 4a ..] the result
+//            lane owns column d0 + (lane & 15) of the keys key0 .. key0 + 3 - half of an MFMA operand's 8 k slots.
+// Requires every byte offset inside a q / k / v plane to fit 32 bits (checked by the caller).
+template <int WS_Y, int WS_X, bool HAS_BIAS>
+struct AttnDmaCfg {
+  static constexpr int L = WS_Y * WS_X;
+  static constexpr int NQ = (L + 31) / 32;
+  static constexpr int LPAD = NQ * 32;
+  static constexpr int NWAVES = (NQ + 1) / 2;
+  static constexpr int NT = NWAVES * 64;
+  static constexpr int TBL = (2 * WS_Y - 1) * (2 * WS_X - 1);
+  static constexpr int KV_BYTES = LPAD * 128;
+  static constexpr int SMEM = 2 * KV_BYTES + (HAS_BIAS ? TBL * 16 : 0);
+};
+
+template <int WS_Y, int WS_X, bool HAS_BIAS>
+__global__ void __launch_bounds__(attn_threads(WS_Y, WS_X)) __attribute__((amdgpu_waves_per_eu(2)))
+window_attention_dma_kernel(AttnParams p) {
+  using Cfg = AttnDmaCfg<WS_Y, WS_X, HAS_BIAS>;
+  constexpr int HD = 64, KS = 4, DB = 2;
+  constexpr int L = Cfg::L, NQ = Cfg::NQ, LPAD = Cfg::LPAD, NT = Cfg::NT, NWAVES = Cfg::NWAVES, TBL = Cfg::TBL;
+  static_assert(WS_X % 4 == 0, "groups of 4 consecutive keys must stay inside one window row");
+  constexpr float LOG2E = 1.4426950408889634f;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char* sK = smem;
+  unsigned char* sV = smem + Cfg::KV_BYTES;
+  unsigned char* sB = smem + 2 * Cfg::KV_BYTES;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l31 = lane & 31, hi = lane >> 5;
+
+  const int head = blockIdx.x % p.heads;
+  const int win = blockIdx.x / p.heads;
+  const int wpi = p.nWy * p.nWx;
+  const int b = win / wpi;
+  const int wrem = win - b * wpi;
+  const int wy = wrem / p.nWx, wx = wrem - wy * p.nWx;
+  const int H = p.H, W = p.W;
+  const int inner = p.heads * HD;
+  const uint32_t ld_qkv = (uint32_t)p.tok_stride;
+  const uint32_t img_base = (uint32_t)b * (uint32_t)(H * W);
+  const int y0 = wy * WS_Y + p.sy, x0 = wx * WS_X + p.sx;
+
+  auto token_row = [&](int pos) -> uint32_t {
+    int Y = y0 + pos / WS_X;
+    int X = x0 + pos % WS_X;
+    if (Y >= H) Y -= H;
+    if (X >= W) X -= W;
+    return img_base + (uint32_t)Y * (uint32_t)W + (uint32_t)X;
+  };
+
+  // ---- K and V: global -> LDS.  Instruction ii fills rows 8 ii .. 8 ii + 7 of both tiles; the waves share them out.
+  {
+    const uint16_t* kbase = p.qkv + p.part_stride + head * p.head_stride;
+    const uint16_t* vbase = p.qkv + 2 * p.part_stride + head * p.head_stride;
+    const uint32_t plane_bytes = (uint32_t)p.B * (uint32_t)(H * W) * ld_qkv * 2u;  // < 2^32, checked by the caller
+    const __amdgpu_buffer_rsrc_t rs_k = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)plane_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_v = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (int)plane_bytes, 0x00020000);
+    const int rsub = lane >> 3, pc = lane & 7;
+#pragma unroll
+    for (int j = 0; j < (LPAD / 8 + NWAVES - 1) / NWAVES; ++j) {
+      const int ii = wave + j * NWAVES;
+      if (ii < LPAD / 8) {  // wave-uniform
+        const int key = ii * 8 + rsub;
+        uint32_t off_k = 0xFFFFFFF0u, off_v = 0xFFFFFFF0u;  // rows past the window: outside the descriptor, arrive as zeros
+        if (LPAD == L || key < L) {
+          const uint32_t row_off = token_row(key) * (ld_qkv * 2u);
+          off_k = row_off + (uint32_t)((pc ^ ((key >> 1) & 7)) << 4);
+          off_v = row_off + (uint32_t)((pc ^ (2 * (key & 3))) << 4);
+        }
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_k, (lds_ptr)(sK + ii * 1024), 16, off_k, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_v, (lds_ptr)(sV + ii * 1024), 16, off_v, 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- Q fragments of both query groups of this wave (B operand): lane = query, 8 consecutive d per k16 step
+  bf16x8 qf[2][KS];
+  uint32_t q_tok[2];
+#pragma unroll
+  for (int ps = 0; ps < 2; ++ps) {
+    int qpos = (wave + ps * NWAVES) * 32 + l31;
+    if (qpos >= L) qpos = L - 1;
+    q_tok[ps] = token_row(qpos);
+    const uint16_t* qp = p.qkv + head * p.head_stride + (uint64_t)q_tok[ps] * ld_qkv + hi * 8;
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) qf[ps][s2] = *reinterpret_cast<const bf16x8*>(qp + s2 * 16);
+  }
+
+  // ---- bias column of this head -> LDS as fp32 4-vectors R4[s] = R[s..s+3] (R reversed, times log2 e)
+  if (HAS_BIAS) {
+    constexpr int BIT = (TBL + NT - 1) / NT;
+    float breg[BIT];
+#pragma unroll
+    for (int it = 0; it < BIT; ++it) {
+      const int j = tid + it * NT;
+      breg[it] = j < TBL ? bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E : 0.f;
+    }
+    float* sBf = reinterpret_cast<float*>(sB);
+#pragma unroll
+    for (int it = 0; it < BIT; ++it) {
+      const int j = tid + it * NT;
+      if (j < TBL) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (j - e >= 0) sBf[(j - e) * 4 + e] = breg[it];
+      }
+    }
+  }
+  // ---- q * scale * log2(e): the accumulators of K Q^T are then the logits in the exp2 domain
+  {
+    const float c = p.scale * LOG2E;
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps)
+#pragma unroll
+      for (int s2 = 0; s2 < KS; ++s2) {
+        u32x4 w = __builtin_bit_cast(u32x4, qf[ps][s2]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(bf16_lo(w[e]) * c, bf16_hi(w[e]) * c);
+        qf[ps][s2] = __builtin_bit_cast(bf16x8, w);
+      }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): this wave's loads into LDS and its bias writes have landed
+  __syncthreads();
+
+  const bool my = p.use_mask && p.sy > 0 && wy == p.nWy - 1;
+  const bool mx = p.use_mask && p.sx > 0 && wx == p.nWx - 1;
+  constexpr float MASK_NEG = -100.0f * LOG2E;
+
+  // per-lane part of the V^T fragment addresses: block of 16 lanes jb = lane >> 4 (column half jb & 1, key half hi = jb >> 1),
+  // source lane 4 e + a inside it
+  uint32_t v_lane[DB];
+  {
+    const int jb = lane >> 4, e = (lane >> 2) & 3, a = lane & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = (4 * db + 2 * (jb & 1) + (a >> 1)) ^ (2 * e);
+      v_lane[db] = (uint32_t)((4 * (jb >> 1) + e) * 128 + (chunk << 4) + (a & 1) * 8);
+    }
+  }
+
+#pragma unroll
+  for (int ps = 0; ps < 2; ++ps) {
+    const int qg = wave + ps * NWAVES;
+    if (qg >= NQ) break;  // wave-uniform
+    int qpos = qg * 32 + l31;
+    const bool q_valid = qpos < L;
+    if (!q_valid) qpos = L - 1;
+    const int qiy = qpos / WS_X, qix = qpos % WS_X;
+    const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
+    const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
+    const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
+
+    auto init_acc = [&](int kb, f32x16& a) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+        if (HAS_BIAS) {
+          const int key0 = kb * 32 + g * 8 + hi * 4;
+          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
+          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
+          bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[g * 4 + i] = bv[i];
+      }
+    };
+    auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
+#pragma unroll
+      for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<64>(kb * 32 + l31, s2 * 2 + hi));
+    };
+    auto mask_block = [&](int kb, f32x16& a) {
+      if (my || mx) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = kb * 32 + g * 8 + hi * 4 + i;
+            const int kiy = key / WS_X, kix = key % WS_X;
+            const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
+            const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
+            if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
+          }
+      }
+      if (LPAD != L) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (kb * 32 + g * 8 + hi * 4 >= L) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[g * 4 + i] = -INFINITY;
+          }
+      }
+    };
+    // V^T fragment of PV step `step`: k slots 0-3 <-> keys 16 step + 4 hi + (0..3), slots 4-7 <-> keys 16 step + 8 + 4 hi + (0..3)
+    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048));
+        const bf16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048 + 1024));
+        f[db] = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+    };
+
+    f32x16 o[DB];
+    float sum;
+    {  // ---- one sweep over the key blocks, P = exp2(logit), range checked afterwards (see window_attention_kernel)
+      f32x16 acc3[3];
+      bf16x8 kf[2][KS], vf[2][DB];
+      uint32_t pk[8];
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+      sum = 0.f;
+      load_k(0, kf[0]);
+      init_acc(0, acc3[0]);
+      if (NQ > 1) {
+        load_k(1, kf[1]);
+        init_acc(1, acc3[1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s2 = 0; s2 < KS; ++s2)
+        acc3[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0][s2], qf[ps][s2], acc3[0], 0, 0, 0);
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb) {
+        f32x16& a = acc3[kb % 3];
+        __builtin_amdgcn_sched_barrier(0);
+        load_v(2 * kb, vf[0]);
+        load_v(2 * kb + 1, vf[1]);
+        if (kb + 1 < NQ) {
+#pragma unroll
+          for (int s2 = 0; s2 < KS; ++s2)
+            acc3[(kb + 1) % 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[(kb + 1) & 1][s2], qf[ps][s2], acc3[(kb + 1) % 3], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (kb + 2 < NQ) {
+          load_k(kb + 2, kf[kb & 1]);
+          init_acc(kb + 2, acc3[(kb + 2) % 3]);
+        }
+        mask_block(kb, a);
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+          const float e0 = __builtin_amdgcn_exp2f(a[2 * h]);
+          const float e1 = __builtin_amdgcn_exp2f(a[2 * h + 1]);
+          pk[h] = pack_bf16x2(e0, e1);
+          sum = dot2_ones(pk[h], sum);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          const u32x4 pw = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
+          const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+          for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t2][db], pf, o[db], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      sum += __shfl_xor(sum, 32, 64);
+    }
+    const bool in_range = sum >= 0x1p-40f && sum <= 0x1p100f;
+    if (__builtin_amdgcn_ballot_w64(!in_range) != 0) {
+      // ---- rows whose logits leave the range: row maximum first (S^T recomputed block by block), then P = exp2(logit - max)
+      float mrow = -INFINITY;
+#pragma unroll 1
+      for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 1) {
+          mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
+          sum = 0.f;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+        }
+#pragma unroll 1
+        for (int kb = 0; kb < NQ; ++kb) {
+          f32x16 a;
+          bf16x8 kf[KS];
+          load_k(kb, kf);
+          init_acc(kb, a);
+#pragma unroll
+          for (int s2 = 0; s2 < KS; ++s2) a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s2], qf[ps][s2], a, 0, 0, 0);
+          mask_block(kb, a);
+          if (pass == 0) {
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) mrow = fmaxf(fmaxf(mrow, a[e]), a[e + 1]);
+          } else {
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+              bf16x8 vf[DB];
+              load_v(2 * kb + t2, vf);
+              uint32_t pk[4];
+#pragma unroll
+              for (int h = 0; h < 4; ++h) {
+                const int h2 = 4 * t2 + h;
+                pk[h] = pack_bf16x2(__builtin_amdgcn_exp2f(a[2 * h2] - mrow), __builtin_amdgcn_exp2f(a[2 * h2 + 1] - mrow));
+                sum = dot2_ones(pk[h], sum);
+              }
+              const u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
+              const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+              for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf, o[db], 0, 0, 0);
+            }
+          }
+        }
+      }
+      sum += __shfl_xor(sum, 32, 64);
+    }
+    const float inv = __builtin_amdgcn_rcpf(sum);
+    {
+      uint16_t* op = p.out + (uint64_t)q_tok[ps] * (uint32_t)inner + head * HD + hi * 8;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          const int g0 = 2 * m, g1 = 2 * m + 1;
+          const uint32_t x0 = pack_bf16x2(o[db][g0 * 4] * inv, o[db][g0 * 4 + 1] * inv);
+          const uint32_t x1 = pack_bf16x2(o[db][g0 * 4 + 2] * inv, o[db][g0 * 4 + 3] * inv);
+          const uint32_t y0 = pack_bf16x2(o[db][g1 * 4] * inv, o[db][g1 * 4 + 1] * inv);
+          const uint32_t y1 = pack_bf16x2(o[db][g1 * 4 + 2] * inv, o[db][g1 * 4 + 3] * inv);
+          const auto rx = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+          const auto ry = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+          if (q_valid) *reinterpret_cast<u32x4*>(op + db * 32 + m * 16) = u32x4{rx[0], ry[0], rx[1], ry[1]};
+        }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Persistent form of the kernel above: one workgroup per CU walks a contiguous range of (head, window) units, one
+// wave per 32-query group, with two K / V buffer sets in LDS.  While the waves compute unit i from one set, the load
+// unit fills the other with unit i + 1 (buffer_load ... lds costs the waves 8 instructions each and no registers), so
+// the HBM stream and the arithmetic overlap inside one workgroup instead of depending on how two independent
+// workgroups on a CU happen to interleave.  One workgroup barrier per unit: a wave passes it when its share of unit
+// i + 1 has landed; everyone having passed it means unit i's buffers are free for unit i + 2.
+// Units are ordered head-major, so a workgroup's consecutive units share the head and its relative-position bias
+// column in LDS is rebuilt only when the head changes.
+template <int WS_Y, int WS_X, bool HAS_BIAS>
+struct AttnPersistCfg {
+  static constexpr int L = WS_Y * WS_X;
+  static constexpr int NQ = (L + 31) / 32;
+  static constexpr int LPAD = NQ * 32;
+  static constexpr int NT = NQ * 64;  // one wave per query group
+  static constexpr int TBL = (2 * WS_Y - 1) * (2 * WS_X - 1);
+  static constexpr int KV_BYTES = LPAD * 128;
+  static constexpr int SMEM = 4 * KV_BYTES + (HAS_BIAS ? TBL * 16 : 0);
+};
+
+constexpr int attn_persist_threads(int ws_y, int ws_x) { return ((ws_y * ws_x + 31) / 32) * 64; }
+
+template <int WS_Y, int WS_X, bool HAS_BIAS>
+__global__ void __launch_bounds__(attn_persist_threads(WS_Y, WS_X))
+window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
+  using Cfg = AttnPersistCfg<WS_Y, WS_X, HAS_BIAS>;
+  constexpr int HD = 64, KS = 4, DB = 2;
+  constexpr int L = Cfg::L, NQ = Cfg::NQ, LPAD = Cfg::LPAD, NT = Cfg::NT, TBL = Cfg::TBL, KVB = Cfg::KV_BYTES;
+  static_assert(WS_X % 4 == 0, "groups of 4 consecutive keys must stay inside one window row");
+  constexpr float LOG2E = 1.4426950408889634f;
+  constexpr int DMA_PER_WAVE = (LPAD / 8 + NQ - 1) / NQ;  // instruction pairs (K, V) per wave and unit
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char* sB = smem + 4 * KVB;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l31 = lane & 31, hi = lane >> 5;
+  const int H = p.H, W = p.W;
+  const int inner = p.heads * HD;
+  const uint32_t ld_qkv = (uint32_t)p.tok_stride;
+  const int wpi = p.nWy * p.nWx;
+  const int n_win = p.B * wpi;
+
+  const int u_begin = blockIdx.x * units_per_wg;
+  int u_end = u_begin + units_per_wg;
+  if (u_end > n_units) u_end = n_units;
+  if (u_begin >= u_end) return;
+
+  const uint32_t plane_bytes = (uint32_t)p.B * (uint32_t)(H * W) * ld_qkv * 2u;  // < 2^32, checked by the caller
+  const int rsub = lane >> 3, pc = lane & 7;
+
+  // A unit = (head, batch entry, window row, window column), walked window-fastest; everything about it is
+  // workgroup-uniform and lives in scalar registers.  The successor of a unit follows by carries, without a division.
+  struct Unit { int head, b, wy, wx; };
+  auto decode = [&](int u) {
+    Unit r;
+    r.head = u / n_win;
+    const int win = u - r.head * n_win;
+    r.b = win / wpi;
+    const int wrem = win - r.b * wpi;
+    r.wy = wrem / p.nWx;
+    r.wx = wrem - r.wy * p.nWx;
+    return r;
+  };
+  auto successor = [&](Unit r) {
+    if (++r.wx == p.nWx) {
+      r.wx = 0;
+      if (++r.wy == p.nWy) {
+        r.wy = 0;
+        if (++r.b == p.B) {
+          r.b = 0;
+          ++r.head;
+        }
+      }
+    }
+    return r;
+  };
+  // Token row of window position (iy, ix): away from the wrapped border (every window of an un-shifted grid, all but
+  // the last window row / column of a shifted one) it is the window's first token plus a per-lane constant; `rel` is
+  // that constant, iy * W + ix.  Windows on the border take the two conditional subtractions.
+  auto window_wraps = [&](const Unit& un) { return (un.wy + 1) * WS_Y + p.sy > H || (un.wx + 1) * WS_X + p.sx > W; };
+  auto window_base = [&](const Unit& un) -> uint32_t {
+    return (uint32_t)un.b * (uint32_t)(H * W) + (uint32_t)(un.wy * WS_Y + p.sy) * (uint32_t)W + (uint32_t)(un.wx * WS_X + p.sx);
+  };
+  auto token_row = [&](const Unit& un, int pos) -> uint32_t {  // general form, used on the border only
+    int Y = un.wy * WS_Y + p.sy + pos / WS_X;
+    int X = un.wx * WS_X + p.sx + pos % WS_X;
+    if (Y >= H) Y -= H;
+    if (X >= W) X -= W;
+    return (uint32_t)un.b * (uint32_t)(H * W) + (uint32_t)Y * (uint32_t)W + (uint32_t)X;
+  };
+  // K and V of unit `un` -> buffer set `set`: instruction pair ii fills rows 8 ii .. 8 ii + 7 of both tiles; a wave
+  // issues pairs wave, wave + NQ, ...  Per pair and lane: key, and the byte offsets of its K / V chunk relative to
+  // the window's first token (un-wrapped windows).
+  uint32_t kv_relk[DMA_PER_WAVE], kv_relv[DMA_PER_WAVE];
+#pragma unroll
+  for (int j = 0; j < DMA_PER_WAVE; ++j) {
+    const int key = (wave + j * NQ) * 8 + rsub;
+    const uint32_t rel = (uint32_t)((key / WS_X) * W + key % WS_X) * (ld_qkv * 2u);
+    kv_relk[j] = rel + (uint32_t)((pc ^ ((key >> 1) & 7)) << 4);
+    kv_relv[j] = rel + (uint32_t)((pc ^ (2 * (key & 3))) << 4);
+  }
+  // The loads of a unit: descriptors and the window's base offset (kv_prepare), then one buffer_load ... lds per
+  // call of kv_issue.  They are issued back to back right after the unit barrier.  (Spreading them over the key-block
+  // loop, one per block, was measured 8 % slower: a load holds the issuing wave while the CU's one address unit
+  // takes its 64 addresses, and inside the loop that wait lands on the arithmetic.)
+  constexpr int N_DMA = 2 * DMA_PER_WAVE;
+  __amdgpu_buffer_rsrc_t kv_rs_k = __builtin_amdgcn_make_buffer_rsrc((void*)p.qkv, 0, 0, 0x00020000);
+  __amdgpu_buffer_rsrc_t kv_rs_v = kv_rs_k;
+  bool kv_wraps = false;
+  uint32_t kv_base = 0;
+  Unit kv_unit = {0, 0, 0, 0};
+  auto kv_prepare = [&](const Unit& un) {
+    const uint16_t* kbase = p.qkv + p.part_stride + un.head * p.head_stride;
+    const uint16_t* vbase = p.qkv + 2 * p.part_stride + un.head * p.head_stride;
+    kv_rs_k = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)plane_bytes, 0x00020000);
+    kv_rs_v = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (int)plane_bytes, 0x00020000);
+    kv_wraps = window_wraps(un);
+    kv_base = window_base(un) * (ld_qkv * 2u);
+    kv_unit = un;
+  };
+  // load number idx of the prepared unit -> buffer set `set`: pair idx / 2 (rows 8 ii .. 8 ii + 7), K for even idx, V for odd
+  auto kv_issue = [&](int idx, int set) {
+    const int j = idx >> 1, is_v = idx & 1;
+    const int ii = wave + j * NQ;  // the pairs divide evenly among the waves for every window built here
+    const int key = ii * 8 + rsub;
+    uint32_t off = kv_base + (is_v ? kv_relv[j] : kv_relk[j]);
+    if (kv_wraps)  // wave-uniform: windows on the wrapped border of a shifted grid
+      off = token_row(kv_unit, key < L ? key : 0) * (ld_qkv * 2u) + (uint32_t)((pc ^ (is_v ? 2 * (key & 3) : (key >> 1) & 7)) << 4);
+    if (LPAD != L && key >= L) off = 0xFFFFFFF0u;  // outside the descriptor: arrives as zeros
+    unsigned char* dst = smem + set * 2 * KVB + is_v * KVB + ii * 1024;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(is_v ? kv_rs_v : kv_rs_k, (lds_ptr)dst, 16, off, 0, 0, 0);
+  };
+  int qpos = wave * 32 + l31;
+  const bool q_valid = qpos < L;
+  if (!q_valid) qpos = L - 1;
+  const int qiy = qpos / WS_X, qix = qpos % WS_X;
+  const uint32_t q_rel = (uint32_t)(qiy * W + qix);
+  // Q fragments of this wave's query group (B operand: lane = query, 8 consecutive d per k16 step)
+  auto load_q = [&](const Unit& un, bf16x8 (&q)[KS], uint32_t& tok) {
+    tok = window_wraps(un) ? token_row(un, qpos) : window_base(un) + q_rel;
+    const uint16_t* qp = p.qkv + un.head * p.head_stride + (uint64_t)tok * ld_qkv + hi * 8;
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) q[s2] = *reinterpret_cast<const bf16x8*>(qp + s2 * 16);
+  };
+  auto build_bias = [&](int head) {
+    if (HAS_BIAS) {
+      float* sBf = reinterpret_cast<float*>(sB);
+      for (int j = tid; j < TBL; j += NT) {
+        const float r = bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E;  // R[j]
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (j - e >= 0) sBf[(j - e) * 4 + e] = r;  // R4[j-e][e] = R[j]
+      }
+    }
+  };
+
+  // per-lane part of the V^T fragment addresses (see window_attention_dma_kernel)
+  uint32_t v_lane[DB];
+  {
+    const int jb = lane >> 4, e = (lane >> 2) & 3, a = lane & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = (4 * db + 2 * (jb & 1) + (a >> 1)) ^ (2 * e);
+      v_lane[db] = (uint32_t)((4 * (jb >> 1) + e) * 128 + (chunk << 4) + (a & 1) * 8);
+    }
+  }
+  const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
+  const float cq = p.scale * LOG2E;
+  constexpr float MASK_NEG = -100.0f * LOG2E;
+
+  Unit cur = decode(u_begin);
+  int bias_head = cur.head;
+  bf16x8 q_cur[KS], q_nxt[KS];
+  uint32_t tok_cur, tok_nxt = 0;
+  static_assert((LPAD / 8) % NQ == 0, "the load pairs must divide evenly among the waves");
+  load_q(cur, q_cur, tok_cur);
+  kv_prepare(cur);
+#pragma unroll
+  for (int i = 0; i < N_DMA; ++i) kv_issue(i, 0);
+  build_bias(bias_head);
+#pragma unroll
+  for (int s2 = 0; s2 < KS; ++s2) q_nxt[s2] = q_cur[s2];
+
+  for (int u = u_begin; u < u_end; ++u) {
+    const int set = (u - u_begin) & 1;
+    const bool more = u + 1 < u_end;
+    const Unit nxt = successor(cur);
+    if (HAS_BIAS && cur.head != bias_head) {  // workgroup-uniform and rare: the range crosses into the next head
+      __syncthreads();
+      build_bias(cur.head);
+      bias_head = cur.head;
+    }
+    // this wave's loads of unit u (and its bias writes) have landed; only the 4 output stores of the unit before may
+    // still be outstanding (vector memory operations complete in order)
+    if (u == u_begin) __builtin_amdgcn_s_waitcnt(0x0070);
+    else __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) {  // Q first: a later wait for it then does not have to wait for the K / V loads behind it
+      load_q(nxt, q_nxt, tok_nxt);
+      kv_prepare(nxt);
+#pragma unroll
+      for (int i = 0; i < N_DMA; ++i) kv_issue(i, set ^ 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const unsigned char* sK = smem + set * 2 * KVB;
+    const unsigned char* sV = sK + KVB;
+    const bool my = p.use_mask && p.sy > 0 && cur.wy == p.nWy - 1;
+    const bool mx = p.use_mask && p.sx > 0 && cur.wx == p.nWx - 1;
+    const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
+    const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
+    bf16x8 qf[KS];
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) {
+      u32x4 w = __builtin_bit_cast(u32x4, q_cur[s2]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(bf16_lo(w[e]) * cq, bf16_hi(w[e]) * cq);
+      qf[s2] = __builtin_bit_cast(bf16x8, w);
+    }
+
+    auto init_acc = [&](int kb, f32x16& a) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+        if (HAS_BIAS) {
+          const int key0 = kb * 32 + g * 8 + hi * 4;
+          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
+          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
+          bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[g * 4 + i] = bv[i];
+      }
+    };
+    auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
+#pragma unroll
+      for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<64>(kb * 32 + l31, s2 * 2 + hi));
+    };
+    auto mask_block = [&](int kb, f32x16& a) {
+      if (my || mx) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = kb * 32 + g * 8 + hi * 4 + i;
+            const int kiy = key / WS_X, kix = key % WS_X;
+            const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
+            const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
+            if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
+          }
+      }
+      if (LPAD != L) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (kb * 32 + g * 8 + hi * 4 >= L) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[g * 4 + i] = -INFINITY;
+          }
+      }
+    };
+    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048));
+        const bf16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048 + 1024));
+        f[db] = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+    };
+
+    f32x16 o[DB];
+    float sum;
+    {
+      // one sweep over the key blocks, P = exp2(logit), range checked afterwards (see window_attention_kernel).  Without
+      // a bias the first MFMA of an S^T block takes a literal zero as its C operand, and so does the first one of O^T:
+      // no accumulator is ever zero-filled by the VALU.
+      const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      f32x16 acc2[2];
+      bf16x8 kf[2][KS], vf[2][DB];
+      uint32_t pk[8];
+      sum = 0.f;
+      auto qk_block = [&](int kb, f32x16& acc, const bf16x8 (&kfr)[KS]) {
+#pragma unroll
+        for (int s2 = 0; s2 < KS; ++s2)
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[s2], qf[s2], (!HAS_BIAS && s2 == 0) ? zero16 : acc, 0, 0, 0);
+      };
+      load_k(0, kf[0]);
+      if (HAS_BIAS) init_acc(0, acc2[0]);
+      if (NQ > 1) {
+        load_k(1, kf[1]);
+        if (HAS_BIAS) init_acc(1, acc2[1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      qk_block(0, acc2[0], kf[0]);
+#pragma unroll
+      for (int kb = 0; kb < NQ; ++kb) {
+        f32x16& a = acc2[kb & 1];
+        __builtin_amdgcn_sched_barrier(0);
+        load_v(2 * kb, vf[0]);
+        load_v(2 * kb + 1, vf[1]);
+        if (kb + 1 < NQ) qk_block(kb + 1, acc2[(kb + 1) & 1], kf[(kb + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kb + 2 < NQ) load_k(kb + 2, kf[kb & 1]);
+        mask_block(kb, a);
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+          const float e0 = __builtin_amdgcn_exp2f(a[2 * h]);
+          const float e1 = __builtin_amdgcn_exp2f(a[2 * h + 1]);
+          pk[h] = pack_bf16x2(e0, e1);
+          sum = dot2_ones(pk[h], sum);  // the row sum of what PV multiplies: the rounded values
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // the accumulators of block kb are consumed: the bias of block kb + 2 goes straight into them
+        if (HAS_BIAS && kb + 2 < NQ) init_acc(kb + 2, a);
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          const u32x4 pw = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
+          const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t2][db], pf, (kb == 0 && t2 == 0) ? zero16 : o[db], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      sum += __shfl_xor(sum, 32, 64);
+    }
+    const bool in_range = sum >= 0x1p-40f && sum <= 0x1p100f;
+    if (__builtin_amdgcn_ballot_w64(!in_range) != 0) {
+      float mrow = -INFINITY;
+#pragma unroll 1
+      for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 1) {
+          mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
+          sum = 0.f;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+        }
+#pragma unroll 1
+        for (int kb = 0; kb < NQ; ++kb) {
+          f32x16 a;
+          bf16x8 kf[KS];
+          load_k(kb, kf);
+          init_acc(kb, a);
+#pragma unroll
+          for (int s2 = 0; s2 < KS; ++s2) a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s2], qf[s2], a, 0, 0, 0);
+          mask_block(kb, a);
+          if (pass == 0) {
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) mrow = fmaxf(fmaxf(mrow, a[e]), a[e + 1]);
+          } else {
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+              bf16x8 vf[DB];
+              load_v(2 * kb + t2, vf);
+              uint32_t pk[4];
+#pragma unroll
+              for (int h = 0; h < 4; ++h) {
+                const int h2 = 4 * t2 + h;
+                pk[h] = pack_bf16x2(__builtin_amdgcn_exp2f(a[2 * h2] - mrow), __builtin_amdgcn_exp2f(a[2 * h2 + 1] - mrow));
+                sum = dot2_ones(pk[h], sum);
+              }
+              const u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
+              const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+              for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf, o[db], 0, 0, 0);
+            }
+          }
+        }
+      }
+      sum += __shfl_xor(sum, 32, 64);
+    }
+    const float inv = __builtin_amdgcn_rcpf(sum);
+    {
+      // Always 4 stores per wave and unit (the wait at the top of the loop counts them); rows past the window store
+      // their (recomputed, identical) last row again.  o[db][4g+i] = O[query][32db + 8g + 4hi + i]: v_permlane32_swap
+      // on the pieces 2m and 2m + 1 gives the lower lane of a query all of piece 2m and the upper lane all of piece
+      // 2m + 1: 32 contiguous bytes per row and instruction.  (64 bytes per row through a further v_permlane16_swap,
+      // and the same for the Q loads, measured no faster.)
+      uint16_t* op = p.out + (uint64_t)tok_cur * (uint32_t)inner + cur.head * HD + hi * 8;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          const int g0 = 2 * m, g1 = 2 * m + 1;
+          const uint32_t x0 = pack_bf16x2(o[db][g0 * 4] * inv, o[db][g0 * 4 + 1] * inv);
+          const uint32_t x1 = pack_bf16x2(o[db][g0 * 4 + 2] * inv, o[db][g0 * 4 + 3] * inv);
+          const uint32_t y0 = pack_bf16x2(o[db][g1 * 4] * inv, o[db][g1 * 4 + 1] * inv);
+          const uint32_t y1 = pack_bf16x2(o[db][g1 * 4 + 2] * inv, o[db][g1 * 4 + 3] * inv);
+          const auto rx = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+          const auto ry = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+          *reinterpret_cast<u32x4*>(op + db * 32 + m * 16) = u32x4{rx[0], ry[0], rx[1], ry[1]};
+        }
+    }
+    cur = nxt;
+    tok_cur = tok_nxt;
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) q_cur[s2] = q_nxt[s2];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 
 #define AERIS_ATTN_SHAPES(X) X(8, 8, 32) X(8, 8, 64) X(12, 12, 32) X(12, 12, 64) X(16, 16, 32) X(16, 16, 64)
+
+static int g_attn_cus = 256;  // compute units of the device (set by attention_configure_all)
 
 bool attention_supported(int ws_y, int ws_x, int head_dim) {
 #define CHK(Y, Xx, D) if (ws_y == Y && ws_x == Xx && head_dim == D) return true;
@@ -463,6 +1214,24 @@ hipError_t attention_configure_all() {
   AERIS_ATTN_SHAPES(CFG)
 #undef CFG
 #undef CFG1
+#define CFGD(Y, Xx, Bi)                                                                                        \
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_dma_kernel<Y, Xx, Bi>),                \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, AttnDmaCfg<Y, Xx, Bi>::SMEM);             \
+  if (e != hipSuccess) return e;
+  CFGD(8, 8, true) CFGD(8, 8, false) CFGD(12, 12, true) CFGD(12, 12, false) CFGD(16, 16, true) CFGD(16, 16, false)
+#undef CFGD
+#define CFGP(Y, Xx, Bi)                                                                                        \
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_persist_kernel<Y, Xx, Bi>),            \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, AttnPersistCfg<Y, Xx, Bi>::SMEM);         \
+  if (e != hipSuccess) return e;
+  CFGP(8, 8, true) CFGP(8, 8, false) CFGP(12, 12, true) CFGP(12, 12, false) CFGP(16, 16, true) CFGP(16, 16, false)
+#undef CFGP
+  {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+        cus > 0)
+      g_attn_cus = cus;
+  }
   return hipSuccess;
 }
 
@@ -470,6 +1239,22 @@ template <int WS_Y, int WS_X, int HD, bool HAS_BIAS>
 static hipError_t launch_attn(const AttnParams& p, hipStream_t stream) {
   using Cfg = AttnCfg<WS_Y, WS_X, HD, HAS_BIAS>;
   const int64_t grid = (int64_t)p.B * p.nWy * p.nWx * p.heads;
+  // head_dim 64 with every offset inside a q / k / v plane below 2^32 bytes: K and V straight into LDS
+  if (HD == 64 && p.head_stride >= (int64_t)p.B * p.H * p.W * p.tok_stride &&
+      (int64_t)p.B * p.H * p.W * p.tok_stride * 2 < (int64_t)0xFFFFFFF0u) {
+    if (grid >= 2 * (int64_t)g_attn_cus) {  // enough units for every CU to stream a few: the persistent form
+      using P = AttnPersistCfg<WS_Y, WS_X, HAS_BIAS>;
+      const int per = (int)((grid + g_attn_cus - 1) / g_attn_cus);
+      const int wgs = (int)((grid + per - 1) / per);
+      hipLaunchKernelGGL((window_attention_persist_kernel<WS_Y, WS_X, HAS_BIAS>), dim3((unsigned)wgs), dim3(P::NT), P::SMEM,
+                         stream, p, per, (int)grid);
+      return hipGetLastError();
+    }
+    using D = AttnDmaCfg<WS_Y, WS_X, HAS_BIAS>;
+    hipLaunchKernelGGL((window_attention_dma_kernel<WS_Y, WS_X, HAS_BIAS>), dim3((unsigned)grid), dim3(D::NT), D::SMEM,
+                       stream, p);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL((window_attention_kernel<WS_Y, WS_X, HD, HAS_BIAS>), dim3((unsigned)grid), dim3(Cfg::NT),
                      Cfg::SMEM, stream, p);
   return hipGetLastError();

@@ -50,7 +50,7 @@ WORKLOADS = {
 }
 
 
-def build_model(pkg, torch, wl, device, residual_dtype):
+def build_model(pkg, torch, wl, device, residual_dtype, init=True):
     ws = wl["window"]
     model = pkg.LocalAERIS(device_mesh=None, heads=wl["heads"], dim=wl["dim"], head_dim=wl["head_dim"],
                            mlp_dim=wl["mlp_dim"], window_size=(ws, ws), image_shape=wl["image_shape"], rope_base=10_000,
@@ -58,6 +58,8 @@ def build_model(pkg, torch, wl, device, residual_dtype):
                            model_in_channels=wl["cin"], model_out_channels=wl["cout"], residual_dtype=residual_dtype,
                            **(dict(preset="ref") if wl.get("preset") == "ref" else dict(preset="spec", mod_ways=2)))
     model = model.to(device)
+    if not init:
+        return model
     g = torch.Generator(device=device).manual_seed(0)
     with torch.no_grad():
         for name, p in model.named_parameters():
@@ -133,34 +135,44 @@ def run_rollout(args, pkg, torch, wl, model, dev):
     print(json.dumps(result))
 
 
-def cpu_baseline(torch, wl, rows, seconds_cap=60.0):
-    """Time the fp32 oracle (this repository's CPU restatement of the reference block) on a strip of the same
-    grid: `rows` lat rows x full longitude, one un-shifted and one shifted block, and scale to a full step."""
+def cpu_baseline_and_parity(pkg, torch, wl, model, rows, dev, residual_dtype):
+    """The CPU leg and the parity figure in one: the fp32 oracle (this repository's CPU restatement of the reference
+    model) runs the WHOLE denoiser - embedding, every block, head - on a strip of the grid, `rows` latitude rows x full
+    longitude, with the benchmarked model's own weights.  Its wall time, scaled by the number of strips in the grid, is
+    the CPU baseline (windows never mix tokens of different window rows, so a strip of whole window rows is a
+    self-contained model run; with one window row the shifted blocks wrap inside it).  The same strip through the HIP
+    model gives relative-L2 and max-abs error of the timed configuration at its full depth."""
     import oracle
     H, W = wl["image_shape"]
     ws = wl["window"]
     threads = torch.get_num_threads()
-    cfg = oracle.OracleConfig.spec(dim=wl["dim"], heads=wl["heads"], head_dim=wl["head_dim"], mlp_dim=wl["mlp_dim"],
-                                   window_size=(ws, ws), image_shape=(rows, W), mod_ways=2)
-    sd = oracle.init_block_weights(cfg, 0)
-    g = torch.Generator().manual_seed(0)
-    x = torch.randn(1, rows * W, wl["dim"], generator=g)
-    t = torch.randn(1, wl["dim"], generator=g)
+    ref = wl.get("preset") == "ref"
+    mk = oracle.OracleConfig.ref if ref else (lambda **kw: oracle.OracleConfig.spec(mod_ways=2, **kw))
+    cfg = mk(dim=wl["dim"], heads=wl["heads"], head_dim=wl["head_dim"], mlp_dim=wl["mlp_dim"], window_size=(ws, ws),
+             image_shape=(rows, W), n_layers=wl["blocks"] + 2, in_channels=wl["cin"], out_channels=wl["cout"])
+    sd = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    strip = build_model(pkg, torch, dict(wl, image_shape=(rows, W)), dev, residual_dtype, init=False)
+    strip.load_state_dict(model.state_dict())
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(1, rows * W, wl["cin"], generator=g)
+    t = torch.rand(1, generator=g) * (math.pi / 2)
     with torch.no_grad():
-        warm = oracle.OracleConfig.spec(dim=wl["dim"], heads=wl["heads"], head_dim=wl["head_dim"], mlp_dim=wl["mlp_dim"],
-                                        window_size=(ws, ws), image_shape=(ws, 4 * ws), mod_ways=2)
-        oracle.block_forward(warm, sd, x[:, :4 * ws * ws], t, (0, 0))  # warm the thread pool and the allocator
+        got = strip(x.to(dev), t.to(dev)).float().cpu()
+        warm = torch.randn(512, 512)
+        (warm @ warm).sum().item()  # spin up the thread pool
         t0 = time.perf_counter()
-        oracle.block_forward(cfg, sd, x, t, (0, 0))
-        t_even = time.perf_counter() - t0
-        t0 = time.perf_counter()
-        oracle.block_forward(cfg, sd, x, t, (ws // 2, ws // 2))
-        t_odd = time.perf_counter() - t0
+        want = oracle.model_forward(cfg, sd, x, t)
+        t_strip = time.perf_counter() - t0
+    del strip
+    diff = (got.double() - want.double())
+    parity = {"rel_l2": float(diff.norm() / want.double().norm()), "max_abs": float(diff.abs().max()),
+              "ref_rms": float(want.double().pow(2).mean().sqrt()), "tolerance_rel_l2": 1e-2,
+              "against": f"fp32 CPU oracle, whole denoiser ({wl['blocks']} blocks) on a {rows}x{W} strip, same weights and inputs"}
     scale = H / rows
-    step_s = (t_even + t_odd) / 2 * wl["blocks"] * scale  # embedding and head (1 % of the FLOPs) left out
-    return {"value": 1.0 / step_s, "unit": "denoise steps/s", "cores": threads, "kind": "port",
-            "sample": f"fp32 torch oracle, one un-shifted + one shifted block on a {rows}x{W} strip "
-                      f"({t_even:.2f}s + {t_odd:.2f}s), scaled x{scale:.1f} rows x{wl['blocks']} blocks (extrapolated)"}
+    base = {"value": 1.0 / (t_strip * scale), "unit": "denoise steps/s", "cores": threads, "kind": "port",
+            "sample": f"fp32 torch oracle, full-depth denoiser forward on a {rows}x{W} strip of the grid: {t_strip:.1f} s, "
+                      f"scaled x{scale:.0f} strips (extrapolated)"}
+    return base, parity
 
 
 def main():
@@ -172,7 +184,8 @@ def main():
     ap.add_argument("--residual", default="f32", choices=["bf16", "f32"],
                     help="dtype of the residual stream between blocks (f32: within 1e-2 of fp32 at 24 blocks; bf16: not)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-rows", type=int, default=96)
+    ap.add_argument("--cpu-rows", type=int, default=0,
+                    help="latitude rows of the strip the CPU oracle runs (a multiple of the window; default: one window row)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -194,6 +207,11 @@ def main():
     wl = WORKLOADS[args.workload]
     H, W = wl["image_shape"]
     S = H * W
+    if args.cpu_rows <= 0:
+        args.cpu_rows = wl["window"]
+    if args.cpu_rows % wl["window"] or H % args.cpu_rows:
+        print("bench.py: --cpu-rows must be a multiple of the window size and divide the grid height", file=sys.stderr)
+        sys.exit(2)
     res_dt = torch.bfloat16 if args.residual == "bf16" else torch.float32
     model = build_model(pkg, torch, wl, dev, res_dt)
     g = torch.Generator(device=dev).manual_seed(1)
@@ -248,13 +266,13 @@ def main():
         byts = 8.0 * S * wl["heads"] * wl["head_dim"]
         k["gbs"] = byts / (k["avg_ms"] * 1e-3) / 1e9
         k["frac_hbm_peak"] = k["gbs"] / PEAK_HBM_GBS
-    NAMES = {"gemm_256x256_none_bf16_res": "gemm_bf16_nt_persistent_kernel<0, false, false, true> (proj / fc2 GEMMs: x gate + residual)",
-             "gemm_256x256_none_bf16": "gemm_bf16_nt_persistent_kernel<0, false, false, false>",
-             "gemm_256x256_none_bf16_plain": "gemm_bf16_nt_persistent_kernel<0, false, true, false> (qkv / embedding GEMMs)",
-             "gemm_256x256_gelu_bf16_plain": "gemm_bf16_nt_persistent_kernel<1, false, true, false> (fc1 GEMM + GELU)",
-             "gemm_256x256_none_f32": "gemm_bf16_nt_persistent_kernel<0, true, false, false>",
-             "gemm_256x256_none_f32_plain": "gemm_bf16_nt_persistent_kernel<0, true, true, false>",
-             "gemm_256x256_swiglu_bf16_plain": "gemm_bf16_nt_persistent_kernel<2, false, true, false>"}
+    NAMES = {"gemm_256x256_none_bf16_res": "gemm_bf16_nt_persistent_kernel<0, false, false, true, false> (proj / fc2 GEMMs on a bf16 residual stream: x gate + residual)",
+             "gemm_256x256_none_bf16": "gemm_bf16_nt_persistent_kernel<0, false, false, false, false>",
+             "gemm_256x256_none_bf16_plain": "gemm_bf16_nt_persistent_kernel<0, false, true, false, false> (qkv GEMM)",
+             "gemm_256x256_gelu_bf16_plain": "gemm_bf16_nt_persistent_kernel<1, false, true, false, false> (fc1 GEMM + GELU)",
+             "gemm_256x256_none_f32": "gemm_bf16_nt_persistent_kernel<0, true, false, false, true> (proj / fc2 GEMMs on the f32 residual stream: x gate + residual)",
+             "gemm_256x256_none_f32_plain": "gemm_bf16_nt_persistent_kernel<0, true, true, false, false> (embedding GEMM)",
+             "gemm_256x256_swiglu_bf16_plain": "gemm_bf16_nt_persistent_kernel<2, false, true, false, false>"}
     big = [t for t in kernels if t.startswith("gemm_256x256")]
     roofline = None
     if big:
@@ -280,8 +298,8 @@ def main():
                               "spec (LayerNorm, scale/shift modulation, rel-pos bias, shift mask, GELU MLP, biases)")},
         "roofline": roofline, "kernels": kernels, "output_finite": finite,
     }
-    if not args.no_cpu_baseline and wl.get("preset") != "ref":  # the CPU leg times the headline block only
-        result["cpu_baseline"] = cpu_baseline(torch, wl, args.cpu_rows)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"], result["parity"] = cpu_baseline_and_parity(pkg, torch, wl, model, args.cpu_rows, dev, res_dt)
         result["gpu_over_cpu"] = result["value"] / result["cpu_baseline"]["value"]
     print(json.dumps(result))
 

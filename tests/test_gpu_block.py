@@ -286,12 +286,13 @@ def test_bench_json_contract_on_a_small_workload(pkg, cuda, monkeypatch, capsys)
     line = [l for l in capsys.readouterr().out.strip().splitlines() if l.startswith("{")][-1]
     r = json.loads(line)
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
-                "vs_baseline", "dtype", "data", "config", "roofline", "kernels", "cpu_baseline"):
+                "vs_baseline", "dtype", "data", "config", "roofline", "kernels", "cpu_baseline", "parity"):
         assert key in r, key
     assert r["n_gpus"] == 1 and r["steps"] == 1 and r["higher_is_better"] is True and r["vs_baseline"] is None
     assert r["value"] > 0 and abs(r["value"] * r["ms_per_step"] - 1000.0) < 1e-6 * 1000.0
     assert "workload" in r["config"] and "model" not in r["config"]
     assert r["output_finite"] is True
+    assert r["parity"]["rel_l2"] <= 1e-2 and r["parity"]["max_abs"] > 0  # the timed model against the oracle, full depth
     cb = r["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and "sample" in cb
     if r["roofline"] is not None:

@@ -163,6 +163,51 @@ def test_window_attention_parity(pkg, cuda, case):
     assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
 
 
+PLANE_CASES = [
+    # B, H, W, heads, hd, ws, shift, bias, mask, magnitude of q and k -- q / k / v as head planes: the kernels that bring
+    # K and V into LDS with buffer_load ... lds and read V^T with the transposing LDS read
+    (1, 160, 160, 24, 64, 16, 8, True, True, 1.0),    # persistent form (2400 units), configs[3] heads
+    (2, 96, 96, 8, 64, 12, 6, True, True, 1.0),       # persistent form, L = 144 padded to 160 (1024 units)
+    (2, 128, 128, 2, 64, 8, 4, True, True, 1.0),      # persistent form, 8x8 windows, two waves per workgroup
+    (1, 160, 160, 24, 64, 16, 0, False, False, 1.0),  # persistent form without bias: accumulators start at a literal zero
+    (3, 32, 48, 2, 64, 16, 8, True, True, 1.0),       # one workgroup per unit (36 units)
+    (1, 36, 48, 3, 64, 12, 6, False, True, 1.0),
+    # logits far outside the range in which exp2 can do without the row maximum: rows take the two-pass form
+    (1, 160, 160, 24, 64, 16, 8, True, True, 6.0),
+    (1, 32, 48, 2, 64, 16, 8, False, False, 8.0),
+    (1, 32, 64, 4, 32, 8, 4, True, True, 8.0),        # head_dim 32: the register-staged kernel, same range check
+]
+
+
+@pytest.mark.parametrize("case", PLANE_CASES, ids=lambda c: f"B{c[0]}_{c[1]}x{c[2]}_h{c[3]}x{c[4]}_ws{c[5]}_s{c[6]}_b{int(c[7])}m{int(c[8])}_x{c[9]:g}")
+def test_window_attention_planes_parity(pkg, cuda, case):
+    B, H, W, heads, hd, ws, sh, has_bias, use_mask, mag = case
+    g = torch.Generator().manual_seed(H * W + heads + int(mag))
+    inner, S = heads * hd, B * H * W
+    qkv = torch.randn(B, H * W, 3 * inner, generator=g)
+    qkv[..., :2 * inner] *= mag  # logits of magnitude mag^2 * sqrt(hd) * scale: up to several hundred, and as far below zero
+    qkv = bf(qkv)
+    table = bf(0.7 * torch.randn((2 * ws - 1) ** 2, heads, generator=g)) if has_bias else None
+    cfg = OracleConfig(dim=inner, heads=heads, head_dim=hd, mlp_dim=inner, window_size=(ws, ws), image_shape=(H, W),
+                       rel_pos_bias=has_bias, shift_mask=use_mask)
+    ref = attention_core(cfg, qkv.float(), (sh, sh), None if table is None else table.float())
+    planes = qkv.view(S, 3 * heads, hd).permute(1, 0, 2).contiguous().to(cuda)  # plane c * heads + h = part c of head h
+    out = pkg.ops.window_attention(planes, B, (H, W), heads, hd, (ws, ws), (sh, sh), None if table is None else table.to(cuda),
+                                   use_mask, head_planes=True)
+    out2 = pkg.ops.window_attention(planes, B, (H, W), heads, hd, (ws, ws), (sh, sh), None if table is None else table.to(cuda),
+                                    use_mask, head_planes=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    assert bool(torch.isfinite(out.float()).all())
+    err = rel_l2(out.view(B, H * W, inner), ref)
+    # P and O are rounded to bf16 once each, and q once more after it is multiplied by the scale (as in the reference,
+    # whose `q * self.scale` is a bf16 product, model.py:290): that rounding moves a logit by 2^-9 of its magnitude,
+    # which is nothing at ordinary magnitudes and a few percent of P once logits reach the hundreds
+    assert err <= (6e-3 if mag == 1.0 else 3e-2), err
+    if mag == 1.0:
+        assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
+
+
 STREAM_CASES = [
     # B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x  -- shapes only the streaming kernel takes
     (1, 120, 120, 2, 128, 60, 60, 30, 30),   # the reference's window: 3600 tokens, head_dim 128 (model.py:22-27), shifted

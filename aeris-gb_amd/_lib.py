@@ -46,6 +46,10 @@ SIGNATURES = {
     "aeris_embed_prepare_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_vp]),
     "aeris_embed_concat_fwd": (_c_int, [_c_vp, _c_int, _c_f32, _c_vp, _c_int, _c_vp, _c_vp, _c_i64, _c_i64, _c_int, _c_int,
                                         _c_vp]),
+    "aeris_input_stage_weight_bytes": (_c_i64, [_c_int, _c_int]),
+    "aeris_input_stage_pack_weight": (_c_int, [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_vp]),
+    "aeris_input_stage_fwd": (_c_int, [_c_vp, _c_int, _c_f32, _c_vp, _c_int, _c_vp, _c_i64, _c_vp, _c_vp, _c_int, _c_i64,
+                                       _c_int, _c_vp]),
 }
 
 _lib = None

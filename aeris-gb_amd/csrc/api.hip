@@ -41,6 +41,7 @@ int ensure_init(void* stream = nullptr, bool from_launch = false) {
     g_init_status = aeris::gemm_configure_all();
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_configure_all();
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_stream_configure_all();
+    if (g_init_status == hipSuccess) g_init_status = aeris::input_stage_configure();
     g_init_done.store(true, std::memory_order_release);
   });
   if (g_init_status == hipSuccess && !from_launch) {
@@ -375,6 +376,43 @@ int aeris_embed_concat_fwd(const float* x0, int C0, float div0, const float* x1,
   hipError_t e = aeris::embed_prepare_launch(x0, C0, div0, x1, C1, ape, out, M, M_ape > 0 ? M_ape : 1, K_pad, split,
                                              reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_embed_concat_fwd launch");
+  return AERIS_OK;
+}
+
+int64_t aeris_input_stage_weight_bytes(int C, int d) {
+  if (!aeris::input_stage_supported(C, d)) return 0;
+  return aeris::input_stage_weight_bytes(C, d);
+}
+
+int aeris_input_stage_pack_weight(const float* W, const float* bias, void* packed, int C, int d, void* stream) {
+  if (!W || !packed) return fail(AERIS_EINVAL, "aeris_input_stage_pack_weight: W/packed is NULL");
+  if (!aeris::input_stage_supported(C, d))
+    return fail(AERIS_EUNSUPPORTED, "aeris_input_stage_pack_weight: need 1 <= C <= 159 and d a multiple of 64 (got C = %d, d = %d)", C, d);
+  if (!aligned16(packed)) return fail(AERIS_EINVAL, "aeris_input_stage_pack_weight: packed must be 16-byte aligned");
+  hipError_t e = aeris::input_stage_pack_weight_launch(W, bias, packed, C, d, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_input_stage_pack_weight launch");
+  return AERIS_OK;
+}
+
+int aeris_input_stage_fwd(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, int64_t M_ape,
+                          const void* packed_w, void* out, int out_dtype, int64_t M, int d, void* stream) {
+  if (!x0 || !packed_w || !out) return fail(AERIS_EINVAL, "aeris_input_stage_fwd: x0/packed_w/out is NULL");
+  if (M <= 0 || C0 <= 0 || C1 < 0 || (x1 == nullptr) != (C1 == 0))
+    return fail(AERIS_EINVAL, "aeris_input_stage_fwd: need M > 0, C0 > 0, and x1 given exactly when C1 > 0");
+  if (!aeris::input_stage_supported(C0 + C1, d))
+    return fail(AERIS_EUNSUPPORTED, "aeris_input_stage_fwd: need C0 + C1 <= 159 and d a multiple of 64 (got C = %d, d = %d)",
+                C0 + C1, d);
+  if (!(div0 != 0.0f)) return fail(AERIS_EINVAL, "aeris_input_stage_fwd: div0 must be non-zero");
+  if (ape && M_ape <= 0) return fail(AERIS_EINVAL, "aeris_input_stage_fwd: M_ape must be positive when ape is given");
+  if (ape && (M_ape < 64 || M_ape > 0x7fffff00))
+    return fail(AERIS_EUNSUPPORTED, "aeris_input_stage_fwd: a positional encoding of fewer than 64 rows (or 2^31 and more) is not "
+                                    "taken (got %lld)", (long long)M_ape);
+  if (out_dtype != AERIS_F32 && out_dtype != AERIS_BF16) return fail(AERIS_EINVAL, "aeris_input_stage_fwd: out_dtype must be f32 or bf16");
+  if (!aligned16(out) || !aligned16(packed_w)) return fail(AERIS_EINVAL, "aeris_input_stage_fwd: out and packed_w must be 16-byte aligned");
+  if (int rc = ensure_init(stream, true)) return rc;
+  hipError_t e = aeris::input_stage_launch(x0, C0, div0, x1, C1, ape, M_ape, packed_w, out, out_dtype, M, d,
+                                           reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_input_stage_fwd launch");
   return AERIS_OK;
 }
 

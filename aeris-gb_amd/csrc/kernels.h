@@ -51,4 +51,13 @@ hipError_t timestep_embedding_launch(const float* t, float* emb, int B, int dim,
 hipError_t embed_prepare_launch(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
                                 int64_t M, int64_t M_ape, int K_pad, int split, hipStream_t stream);
 
+
+// Fused input embedding (input_stage.hip): tokens = ([x0 / div0 | x1] + ape) W^T + b at fp32 accuracy
+bool input_stage_supported(int C, int d);
+int64_t input_stage_weight_bytes(int C, int d);
+hipError_t input_stage_configure();
+hipError_t input_stage_pack_weight_launch(const float* W, const float* bias, void* packed, int C, int d, hipStream_t stream);
+hipError_t input_stage_launch(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, int64_t M_ape,
+                              const void* packed, void* out, int out_dtype, int64_t M, int d, hipStream_t stream);
+
 }  // namespace aeris

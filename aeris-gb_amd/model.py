@@ -270,8 +270,13 @@ class SwinLayer(nn.Module):
             return (self.window_size[0] // 2, self.window_size[1] // 2)
         return (0, 0)
 
-    def block_forward(self, j, x, dt, shift, out=None, branches=None):
-        """One block.  x is not modified; the result is written to ``out`` (allocated if None)."""
+    def block_forward(self, j, x, dt, shift, out=None, tap=None):
+        """One block.  x is not modified; the result is written to ``out`` (allocated if None).
+
+        ``tap(name, tensor, block)``, if given, is shown the two intermediates the block holds anyway before they are
+        consumed: "attn" (attention output ahead of the wo projection) and "hidden" (activated MLP hidden ahead of the
+        down projection), both as views of shared scratch that the next kernel overwrites.
+        """
         o = self.opts
         mods = self.modulelist[j]
         n1, attn, n2, ff = mods[0], mods[1], mods[2], mods[3]
@@ -287,8 +292,8 @@ class SwinLayer(nn.Module):
         # intermediates live in shared scratch buffers (ops.workspace); only `out` is returned
         y = _norm_call(o, n1, x, s1, c1, out=ops.workspace("norm", (b, n, d), torch.bfloat16, x.device))
         a = attn.core(y, shift, out=ops.workspace("attn", (b * n, attn.wo.weight.shape[1]), torch.bfloat16, x.device))
-        if branches is not None:
-            branches["attn"] = ops.gemm(a, attn.wo.weight, attn.wo.bias).view(b, n, d)
+        if tap is not None:
+            tap("attn", a, mods)
         if out is None:
             out = torch.empty_like(x)
         ops.gemm(a, attn.wo.weight, attn.wo.bias, gate=g1, residual=x, rows_per_batch=n, out=out)
@@ -301,12 +306,12 @@ class SwinLayer(nn.Module):
             h = ops.gemm(z, ff.fc1.weight, ff.fc1.bias, act="gelu",
                          out=ops.workspace("hidden", (b, n, ff.fc1.weight.shape[0]), torch.bfloat16, x.device))
             w_dn, b_dn = ff.fc2.weight, ff.fc2.bias
-        if branches is not None:
-            branches["mlp"] = ops.gemm(h, w_dn, b_dn).view(b, n, d)
+        if tap is not None:
+            tap("hidden", h, mods)
         ops.gemm(h, w_dn, b_dn, gate=g2, residual=out, rows_per_batch=n, out=out)  # in place: out += gate * mlp
         return out
 
-    def forward(self, x, dt=None, shift=None, branches=None):
+    def forward(self, x, dt=None, shift=None, tap=None):
         if self.opts.mod_ways and dt is None:
             raise ValueError("this layer is modulated: dt (noise-level embedding [1|b, d]) is required")
         shift = self.default_shift() if shift is None else shift
@@ -314,7 +319,7 @@ class SwinLayer(nn.Module):
             raise TypeError("x must be bf16 or f32")
         x = x.contiguous()
         for j in range(self.sublayers):
-            x = self.block_forward(j, x, dt, shift, branches=branches)
+            x = self.block_forward(j, x, dt, shift, tap=tap)
         return x
 
 
@@ -322,10 +327,12 @@ class InputStage(nn.Module):
     """(+APE) -> Linear(Cin -> d) ; sinusoidal noise-level embedding  (model.py:327-356).
 
     Parameters stay f32 like the reference's, and so does the accuracy of the Linear (fp32 in the reference,
-    model.py:352): the input and the weight are each split into a bf16 head and a bf16 remainder, and one bf16 GEMM
-    over [x_hi | x_lo | x_hi | 1 | 1] x [W_hi | W_hi | W_lo | b_hi | b_lo] sums the three significant products and the
-    bias in fp32 (K = 3 Cin + 2, zero-padded to a multiple of 64).  The split weight is cached and refreshed whenever
-    the parameter changes.
+    model.py:352): the input and the weight are each split into a bf16 head and a bf16 remainder and the three
+    significant products are summed in fp32 on the matrix cores.  One kernel reads the input channels and the
+    positional encoding and writes the token rows (ops.input_stage); shapes it does not take (more than 159 input
+    channels, dim not a multiple of 64) go through an operand matrix [x_hi | x_lo | x_hi | 1 | 1] and one bf16 GEMM
+    against [W_hi | W_hi | W_lo | b_hi | b_lo].  The split weight is cached and refreshed whenever the parameter
+    changes.
     """
 
     def __init__(self, model_in_channels, dim, sinusoidal_emb_max_period, data_dtype=torch.float32,
@@ -339,19 +346,22 @@ class InputStage(nn.Module):
         self.ape_generated = None
         self._wcache = None
 
-    def _weights(self):
+    def _weights(self, fused):
         w, b = self.proj.weight, self.proj.bias
-        key = (w.data_ptr(), w._version, b.data_ptr(), b._version, w.device)
+        key = (w.data_ptr(), w._version, b.data_ptr(), b._version, w.device, fused)
         if self._wcache is None or self._wcache[0] != key:
             c = self.model_in_channels
-            k_pad = (3 * c + 2 + 63) // 64 * 64
-            w32, b32 = w.detach().float(), b.detach().float()
-            w_hi, b_hi = w32.to(torch.bfloat16), b32.to(torch.bfloat16)
-            w_lo, b_lo = (w32 - w_hi.float()).to(torch.bfloat16), (b32 - b_hi.float()).to(torch.bfloat16)
-            wp = torch.zeros(w.shape[0], k_pad, dtype=torch.bfloat16, device=w.device)
-            wp[:, :c], wp[:, c:2 * c], wp[:, 2 * c:3 * c] = w_hi, w_hi, w_lo
-            wp[:, 3 * c], wp[:, 3 * c + 1] = b_hi, b_lo
-            self._wcache = (key, wp, k_pad)
+            w32, b32 = w.detach().float().contiguous(), b.detach().float().contiguous()
+            if fused:
+                self._wcache = (key, ops.input_stage_pack_weight(w32, b32), 0)
+            else:
+                k_pad = (3 * c + 2 + 63) // 64 * 64
+                w_hi, b_hi = w32.to(torch.bfloat16), b32.to(torch.bfloat16)
+                w_lo, b_lo = (w32 - w_hi.float()).to(torch.bfloat16), (b32 - b_hi.float()).to(torch.bfloat16)
+                wp = torch.zeros(w.shape[0], k_pad, dtype=torch.bfloat16, device=w.device)
+                wp[:, :c], wp[:, c:2 * c], wp[:, 2 * c:3 * c] = w_hi, w_hi, w_lo
+                wp[:, 3 * c], wp[:, 3 * c + 1] = b_hi, b_lo
+                self._wcache = (key, wp, k_pad)
         return self._wcache[1:]
 
     def forward(self, x, interval, out_dtype=None, cond=None, x_div=1.0):
@@ -367,13 +377,20 @@ class InputStage(nn.Module):
             ape = ape.reshape(-1, c)
             if ape.shape[0] != n:
                 raise ValueError(f"ape_generated covers {ape.shape[0]} tokens, input has {n}")
-        wp, k_pad = self._weights()
-        if cond is None:
-            a = ops.embed_prepare(x.reshape(b * n, c).float().contiguous(), ape, k_pad, split=True)
+        dim = self.proj.weight.shape[0]
+        fused = ops.input_stage_supported(c, dim) and (ape is None or ape.shape[0] >= 64)
+        wp, k_pad = self._weights(fused)
+        x2 = x.reshape(b * n, -1).float().contiguous()
+        c2 = None if cond is None else cond.reshape(b * n, -1).float().contiguous()
+        if fused:
+            tok = ops.input_stage(x2, x_div if cond is not None else 1.0, c2, ape, wp, dim,
+                                  out_dtype=out_dtype or self.model_dtype).view(b, n, -1)
         else:
-            a = ops.embed_concat(x.reshape(b * n, -1).float().contiguous(), x_div,
-                                 cond.reshape(b * n, -1).float().contiguous(), ape, k_pad, split=True)
-        tok = ops.gemm(a, wp, None, out_dtype=out_dtype or self.model_dtype).view(b, n, -1)
+            if cond is None:
+                a = ops.embed_prepare(x2, ape, k_pad, split=True)
+            else:
+                a = ops.embed_concat(x2, x_div, c2, ape, k_pad, split=True)
+            tok = ops.gemm(a, wp, None, out_dtype=out_dtype or self.model_dtype).view(b, n, -1)
         t = timestep_embedding(interval, tok.shape[-1], self.sinusoidal_emb_max_period)
         return tok, t
 

@@ -404,3 +404,59 @@ def embed_concat(x0: torch.Tensor, div0: float, x1: torch.Tensor, ape: Optional[
     L.call("aeris_embed_concat_fwd", x0.data_ptr(), C0, float(div0), x1.data_ptr(), C1, _ptr(ape), out.data_ptr(), M,
            m_ape, k_pad, int(split), _stream())
     return out
+
+
+def input_stage_supported(C: int, d: int) -> bool:
+    """Whether the one-pass input embedding takes Linear(C -> d) (C <= 159 channels, d a multiple of 64)."""
+    return int(L.lib().aeris_input_stage_weight_bytes(int(C), int(d))) > 0
+
+
+def input_stage_pack_weight(w: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """The packed split-bf16 form of Linear(C -> d)'s f32 parameters that ``input_stage`` multiplies by."""
+    _dev(w, "w", torch.float32)
+    d, C = w.shape
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() != d:
+            raise RuntimeError(f"bias must have {d} elements")
+    nbytes = int(L.lib().aeris_input_stage_weight_bytes(C, d))
+    if nbytes <= 0:
+        raise RuntimeError(f"the one-pass input embedding does not take C = {C}, d = {d}")
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    L.call("aeris_input_stage_pack_weight", w.data_ptr(), _ptr(bias), packed.data_ptr(), C, d, _stream())
+    return packed
+
+
+def input_stage(x0: torch.Tensor, div0: float, x1: Optional[torch.Tensor], ape: Optional[torch.Tensor],
+                packed_w: torch.Tensor, d: int, out_dtype: torch.dtype = torch.float32,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out [M, d] = ([x0 f32 [M, C0] / div0 | x1 f32 [M, C1]] + ape f32 [M_ape, C0 + C1]) W^T + b in one kernel, fp32
+    accuracy; ``packed_w`` from ``input_stage_pack_weight``."""
+    _dev(x0, "x0", torch.float32)
+    C0 = x0.shape[-1]
+    M = x0.numel() // C0
+    C1 = 0
+    if x1 is not None:
+        _dev(x1, "x1", torch.float32)
+        C1 = x1.shape[-1]
+        if x1.numel() // C1 != M:
+            raise RuntimeError("x0 and x1 must have the same number of rows")
+    m_ape = 0
+    if ape is not None:
+        _dev(ape, "ape", torch.float32)
+        m_ape = ape.numel() // (C0 + C1)
+        if ape.shape[-1] != C0 + C1 or M % m_ape:
+            raise RuntimeError("ape must be [M_ape, C0 + C1] with M a multiple of M_ape")
+    need = int(L.lib().aeris_input_stage_weight_bytes(C0 + C1, d))
+    if need <= 0 or packed_w.numel() * packed_w.element_size() != need:
+        raise RuntimeError(f"packed_w does not fit C = {C0 + C1}, d = {d}")
+    if out is None:
+        out = torch.empty(M, d, dtype=out_dtype, device=x0.device)
+    else:
+        _dev(out, "out")
+        if out.numel() != M * d or out.dtype not in (torch.float32, torch.bfloat16):
+            raise RuntimeError("out must be f32 or bf16 [M, d]")
+    with _timed("input_stage", float(M) * ((C0 + C1) * 4 * (2 if ape is not None else 1) + d * out.element_size()), "byte"):
+        L.call("aeris_input_stage_fwd", x0.data_ptr(), C0, float(div0), _ptr(x1), C1, _ptr(ape), m_ape, packed_w.data_ptr(),
+               out.data_ptr(), _DT[out.dtype], M, d, _stream())
+    return out

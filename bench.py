@@ -271,7 +271,8 @@ def main():
              "gemm_256x256_none_bf16_plain": "gemm_bf16_nt_persistent_kernel<0, false, true, false, false> (qkv GEMM)",
              "gemm_256x256_gelu_bf16_plain": "gemm_bf16_nt_persistent_kernel<1, false, true, false, false> (fc1 GEMM + GELU)",
              "gemm_256x256_none_f32": "gemm_bf16_nt_persistent_kernel<0, true, false, false, true> (proj / fc2 GEMMs on the f32 residual stream: x gate + residual)",
-             "gemm_256x256_none_f32_plain": "gemm_bf16_nt_persistent_kernel<0, true, true, false, false> (embedding GEMM)",
+             "gemm_256x256_none_f32_plain": "gemm_bf16_nt_persistent_kernel<0, true, true, false, false> (plain GEMM with f32 output)",
+             "input_stage": "input_stage_kernel<5, true> (concatenation, positional encoding and embedding Linear in one pass)",
              "gemm_256x256_swiglu_bf16_plain": "gemm_bf16_nt_persistent_kernel<2, false, true, false, false>"}
     big = [t for t in kernels if t.startswith("gemm_256x256")]
     roofline = None

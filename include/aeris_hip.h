@@ -188,6 +188,20 @@ int aeris_embed_prepare_fwd(const float* x, const float* ape, void* out, int64_t
 int aeris_embed_concat_fwd(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape, void* out,
                            int64_t M, int64_t M_ape, int K_pad, int split, void* stream);
 
+/* Input embedding in one pass (model.py:346-356; inference.py:160 for the two-part input):
+ *   out [M, d] = ([x0 f32 [M, C0] / div0 | x1 f32 [M, C1]] + ape f32 [M_ape, C0 + C1] or NULL) W^T + b
+ * at the accuracy of the reference's fp32 Linear (inputs and weight each split into bf16 head + remainder, three bf16
+ * MFMA products summed in fp32; about 2^-16 relative), without an [M, K] operand matrix in memory.  x1 may be NULL
+ * with C1 = 0; ape row = m % M_ape; out is f32 or bf16 (out_dtype).  C0 + C1 <= 159, d a multiple of 64, and
+ * M_ape >= 64 when ape is given; other shapes return AERIS_EUNSUPPORTED (use aeris_embed_prepare_fwd / aeris_embed_concat_fwd + aeris_gemm_fwd).
+ * The weight is packed once per parameter value: aeris_input_stage_weight_bytes(C, d) bytes (0 if the shape is not
+ * supported), filled by aeris_input_stage_pack_weight from W f32 [d, C] and b f32 [d] (or NULL). */
+int64_t aeris_input_stage_weight_bytes(int C, int d);
+int aeris_input_stage_pack_weight(const float* W, const float* bias, void* packed, int C, int d, void* stream);
+int aeris_input_stage_fwd(const float* x0, int C0, float div0, const float* x1, int C1, const float* ape,
+                          int64_t M_ape, const void* packed_w, void* out, int out_dtype, int64_t M, int d,
+                          void* stream);
+
 #ifdef __cplusplus
 }
 #endif

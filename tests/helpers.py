@@ -40,3 +40,19 @@ def make_model(pkg, cfg: OracleConfig, sd, device, residual_dtype=torch.bfloat16
     full["input_stage.ape.inv_freq"] = m.state_dict()["input_stage.ape.inv_freq"]
     m.load_state_dict(full, strict=True)
     return m.to(device)
+
+
+def branch_tap(pkg, store):
+    """A ``tap`` for ``SwinLayer.forward`` that projects the two intermediates the block shows it (attention output,
+    activated hidden) without gate or residual, into ``store["attn"]`` / ``store["mlp"]`` - the un-gated branch outputs
+    the oracle returns with ``return_branches=True``."""
+    ops = pkg.ops
+
+    def tap(name, t, mods):
+        if name == "attn":
+            store["attn"] = ops.gemm(t, mods[1].wo.weight, mods[1].wo.bias)
+        else:
+            ff = mods[3]
+            w, b = (ff.w2.weight, None) if hasattr(ff, "w2") else (ff.fc2.weight, ff.fc2.bias)
+            store["mlp"] = ops.gemm(t.reshape(-1, t.shape[-1]), w, b)
+    return tap

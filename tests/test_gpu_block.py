@@ -11,7 +11,7 @@ import torch
 
 import oracle
 from oracle import OracleConfig
-from helpers import make_layer, make_model, rel_l2, max_abs
+from helpers import branch_tap, make_layer, make_model, rel_l2, max_abs
 
 pytestmark = pytest.mark.gpu
 
@@ -31,10 +31,10 @@ def _run_block(pkg, cuda, cfg, seed, nontrivial, shifted, x_dtype=torch.bfloat16
     ref, ref_a, ref_m = oracle.block_forward(cfg, sd, xin.float(), t, shift, return_branches=True)
     layer = make_layer(pkg, cfg, sd, cuda, shifted)
     br = {}
-    out = layer(xin.to(cuda), None if t is None else t.to(cuda), branches=br)
+    out = layer(xin.to(cuda), None if t is None else t.to(cuda), tap=branch_tap(pkg, br))
     torch.cuda.synchronize()
     assert out.dtype == x_dtype and out.shape == x.shape
-    return rel_l2(out, ref), rel_l2(br["attn"], ref_a), rel_l2(br["mlp"], ref_m)
+    return rel_l2(out, ref), rel_l2(br["attn"].view_as(ref_a), ref_a), rel_l2(br["mlp"].view_as(ref_m), ref_m)
 
 
 @pytest.mark.parametrize("shifted", [False, True])

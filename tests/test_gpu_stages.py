@@ -59,6 +59,56 @@ def test_input_stage_alone(pkg, cuda, out_dtype):
     assert rel_l2(tok3, want) > 1e-2  # the encoding is live
 
 
+@pytest.mark.parametrize("case", [
+    # (M, M_ape, C0, C1, d, div0, bias, out dtype)
+    (4096, 2048, 69, 69, 1536, 0.5, True, torch.float32),    # the sampler's form, two batch entries share the encoding
+    (2048, 2048, 138, 0, 1536, 1.0, True, torch.bfloat16),   # plain input, bf16 tokens
+    (1000, 0, 20, 11, 256, 2.0, True, torch.float32),        # ragged rows (1000 = 3 x 256 + 232), one k-step, no encoding
+    (777, 259, 40, 23, 64, 1.0, False, torch.float32),       # encoding wraps inside a workgroup, no bias, two k-steps
+    (300, 100, 96, 0, 128, 3.0, True, torch.float32),        # C = 96: the bias column opens a fourth k-step
+    (256, 256, 159, 0, 192, 1.0, True, torch.float32),       # the widest input the kernel takes
+], ids=["sampler", "plain_bf16", "ragged_small", "wrap_nobias", "k96", "k159"])
+def test_input_stage_kernel_against_float64(pkg, cuda, case):
+    """ops.input_stage (one kernel: channel concatenation, division, positional encoding, Linear + bias) against the
+    same arithmetic in float64.  The reference computes this Linear in fp32 (model.py:350-352)."""
+    M, M_ape, C0, C1, d, div0, with_bias, out_dtype = case
+    ops = pkg.ops
+    g = torch.Generator().manual_seed(M + d)
+    C = C0 + C1
+    x0 = torch.randn(M, C0, generator=g) * 3.0
+    x1 = torch.randn(M, C1, generator=g) if C1 else None
+    ape = torch.rand(M_ape, C, generator=g) * 2.0 - 1.0 if M_ape else None
+    w = torch.randn(d, C, generator=g) * 0.1
+    b = torch.randn(d, generator=g) if with_bias else None
+    assert ops.input_stage_supported(C, d)
+    packed = ops.input_stage_pack_weight(w.to(cuda), None if b is None else b.to(cuda))
+    got = ops.input_stage(x0.to(cuda), div0, None if x1 is None else x1.to(cuda), None if ape is None else ape.to(cuda),
+                          packed, d, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    xin = (x0 / div0).double()
+    if x1 is not None:
+        xin = torch.cat([xin, x1.double()], dim=1)
+    if ape is not None:
+        xin = xin + ape.double().repeat(-(-M // M_ape), 1)[:M]
+    want = xin @ w.double().t() + (0 if b is None else b.double())
+    e, ma = rel_l2(got, want), max_abs(got, want)
+    print(f"input stage kernel {case[:5]}: rel-L2 {e:.3e}, max-abs {ma:.3e}")
+    assert got.dtype == out_dtype and tuple(got.shape) == (M, d)
+    assert e <= (1e-5 if out_dtype == torch.float32 else 3e-3), (e, ma)
+
+
+def test_input_stage_falls_back_for_wide_inputs(pkg, cuda):
+    """More than 159 input channels: the operand-matrix + GEMM form, same accuracy."""
+    ops = pkg.ops
+    assert not ops.input_stage_supported(200, 256) and not ops.input_stage_supported(64, 200)
+    stage = pkg.InputStage(200, 256, 10000.0).to(cuda)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(1, 512, 200, generator=g)
+    tok, _ = stage(x.to(cuda), torch.tensor([0.3], device=cuda), out_dtype=torch.float32)
+    want = x.double() @ stage.proj.weight.detach().double().cpu().t() + stage.proj.bias.detach().double().cpu()
+    assert rel_l2(tok, want) <= 2e-5, rel_l2(tok, want)
+
+
 @pytest.mark.parametrize("preset", ["ref", "spec"])
 @pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16], ids=["f32_stream", "bf16_stream"])
 def test_output_stage_alone(pkg, cuda, preset, x_dtype):

@@ -138,8 +138,29 @@ def test_argument_validation_needs_no_gpu(pkg):
     assert lib.aeris_embed_concat_fwd(p16, 69, 1.0, p16, 69, None, p16, 4, 0, 384, 1, None) == L.EINVAL  # split: too narrow
     assert lib.aeris_embed_concat_fwd(p16, 69, 0.0, p16, 69, None, p16, 4, 0, 192, 0, None) == L.EINVAL  # div0 == 0
     assert lib.aeris_embed_concat_fwd(p16, 69, 1.0, None, 69, None, p16, 4, 0, 192, 0, None) == L.EINVAL  # x1 NULL
+    # fused input stage
+    isw, isp, isf = lib.aeris_input_stage_weight_bytes, lib.aeris_input_stage_pack_weight, lib.aeris_input_stage_fwd
+    assert isw(138, 1536) == 96 * 5 * 2048 and isw(31, 64) == 4 * 1 * 2048 and isw(32, 64) == 4 * 2 * 2048
+    assert isw(160, 1536) == 0 and isw(138, 1500) == 0 and isw(0, 64) == 0  # unsupported shapes: no size
+    assert isp(None, None, p16, 138, 1536, None) == L.EINVAL and isp(p16, None, p16, 160, 1536, None) == L.EUNSUPPORTED
+    ok = (p16, 69, 1.0, p16, 69, None, 0, p16, p16, L.F32, 256, 1536, None)
+    assert isf(*with_of(ok, 0, None)) == L.EINVAL and isf(*with_of(ok, 7, None)) == L.EINVAL  # x0 / packed NULL
+    assert isf(*with_of(ok, 3, None)) == L.EINVAL  # C1 > 0 without x1
+    assert isf(*with_of(ok, 2, 0.0)) == L.EINVAL  # div0 == 0
+    assert isf(*with_of(ok, 1, 100)) == L.EUNSUPPORTED and isf(*with_of(ok, 11, 1500)) == L.EUNSUPPORTED
+    assert isf(*with_of(ok, 10, 0)) == L.EINVAL and isf(*with_of(ok, 9, 7)) == L.EINVAL  # M, out dtype
+    a = list(ok); a[5] = p16; a[6] = 0
+    assert isf(*a) == L.EINVAL  # ape without rows
+    a[6] = 32
+    assert isf(*a) == L.EUNSUPPORTED and "positional" in L.last_error()
     with pytest.raises(pkg.AerisError):
         L.call("aeris_window_index_map", 1, 10, 8, 4, 4, 0, 0, p)
+
+
+def with_of(args, i, v):
+    a = list(args)
+    a[i] = v
+    return a
 
 
 def test_ops_refuse_cpu_tensors(pkg):

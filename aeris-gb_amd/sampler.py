@@ -65,6 +65,7 @@ class _Rollout:
             self.latents = latents.to(dev, torch.float32).contiguous()
         self.B = B
         self.graph, self.step = None, None
+        self._done = 0
         self.reset()
 
     def reset(self):
@@ -72,10 +73,15 @@ class _Rollout:
         self.cond.copy_(self._cond0)
         torch.addcmul(self.x_mean, self.cond, self.x_std, out=self.x_un)
         self.k.zero_()
+        self._done = 0  # host-side mirror of k: the device-side indexing is never asked for a step that does not exist
 
     def run(self, n: Optional[int] = None):
-        """Advance by ``n`` forecast steps (default: all that remain are assumed to be n_forecast) -> states."""
-        for _ in range(self.n_forecast if n is None else n):
+        """Advance by ``n`` forecast steps (default: all that remain) -> the states tensor [n_forecast, B, S, C]."""
+        n = self.n_forecast - self._done if n is None else n
+        if n < 0 or self._done + n > self.n_forecast:
+            raise ValueError(f"{self._done} of {self.n_forecast} forecast steps are done; cannot run {n} more (reset() first)")
+        self._done += n
+        for _ in range(n):
             if self.graph is not None:
                 self.graph.replay()
             else:
@@ -184,6 +190,8 @@ class TrigFlowSampler:
         """Set up an autoregressive forecast (arguments: see ``rollout``) and, with ``use_graph``, capture its
         forecast step (after ``graph_warmup`` eager steps, whose effect on the state is undone).  ``run()`` of the
         returned object advances it; ``reset()`` puts it back to ``state0`` and step 0."""
+        if not 0 <= graph_warmup <= n_forecast:
+            raise ValueError(f"graph_warmup must lie in 0..{n_forecast} (the warm-up steps are forecast steps)")
         ro = _Rollout(state0, n_forecast, x_mean, x_std, t_mean, t_std, forcing, static, extra_cond, latents)
         if use_graph and generator is None and latents is None:
             generator = torch.cuda.default_generators[state0.device.index or 0]

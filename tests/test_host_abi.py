@@ -252,3 +252,23 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
     assert r.returncode == 2
     assert "ONE GPU" in (r.stdout + r.stderr)
+
+
+def test_rollout_refuses_steps_beyond_the_forecast(pkg):
+    """The forecast-step counter lives on the device; the host-side mirror keeps run() from indexing forcings,
+    latents or the state store past their end."""
+    import importlib
+    sm = importlib.import_module(pkg.__name__ + ".sampler")
+    ro = sm._Rollout(torch.zeros(1, 4, 3), 2, None, None, None, None, None, None, None, None)
+    calls = []
+    ro.step = lambda: calls.append(1)
+    ro.run(1)
+    ro.run()
+    assert len(calls) == 2
+    with pytest.raises(ValueError, match="forecast steps are done"):
+        ro.run(1)
+    ro.reset()
+    ro.run(2)
+    assert len(calls) == 4
+    with pytest.raises(ValueError):
+        sm._Rollout(torch.zeros(1, 4, 3), 2, None, None, None, None, torch.zeros(2, 1, 4, 1), None, None, None)  # forcing too short

@@ -20,6 +20,7 @@
 // into that XCD's L2 once and re-read from there by the other query blocks.
 #include "common.h"
 #include "kernels.h"
+#include <type_traits>
 
 namespace aeris {
 
@@ -86,6 +87,7 @@ window_attention_stream_kernel(StreamParams p) {
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   int* tok = reinterpret_cast<int*>(smem + Cfg::TBL_OFF);  // token row (inside the image) of every window position
+  int* const redo = tok + ((p.ws_y * p.ws_x + 3) & ~3);    // set by a wave whose sums left the range of the fast sweep
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l31 = lane & 31, hi = lane >> 5;
@@ -115,6 +117,7 @@ window_attention_stream_kernel(StreamParams p) {
     if (X >= W) X -= W;
     tok[pos] = Y * W + X;
   }
+  if (tid == 0) *redo = 0;
   __syncthreads();
 
   // ---- Q fragments (B operand): lane = query, 8 consecutive d per k16 step
@@ -127,6 +130,19 @@ window_attention_stream_kernel(StreamParams p) {
     const uint16_t* qp = p.qkv + head * p.head_stride + (uint64_t)(uint32_t)q_row * ld_qkv + hi * 8;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
+  }
+  {
+    // q is multiplied by scale * log2(e) once, here (the reference scales q in bf16 too, model.py:290): the
+    // accumulators of K Q^T are then the logits in the exp2 domain and no score needs a multiply
+    const float c = p.scale * LOG2E;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const u32x4 w = __builtin_bit_cast(u32x4, qf[s]);
+      u32x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = pack_bf16x2(bf16_lo(w[e]) * c, bf16_hi(w[e]) * c);
+      qf[s] = __builtin_bit_cast(bf16x8, r);
+    }
   }
 
   const uint16_t* kbase = p.qkv + img_base * (int64_t)ld_qkv + p.part_stride + head * p.head_stride;
@@ -194,9 +210,19 @@ window_attention_stream_kernel(StreamParams p) {
   uint32_t vt_x[4];
 #pragma unroll
   for (int sx = 0; sx < 4; ++sx) vt_x[sx] = (uint32_t)(((2 * sx) ^ hi ^ ((l31 >> 1) & 7) ^ (l31 >> 4)) << 4);
-  const float c = p.scale * LOG2E;
   float m = -INFINITY, l = 0.f;
   f32x16 o[DB];
+  // A wave whose 32 queries all lie past the window (last query block of a window whose size is not a multiple of 256)
+  // only stages K / V and keeps the barriers; its MFMA and softmax work would be thrown away.
+  const bool wave_active = qb * QB + wave * 32 < L;  // wave-uniform
+
+  // One pass over the window's keys.  FAST: P = exp2(logit) without a row maximum - softmax does not depend on the
+  // subtracted constant, the maximum only guards the range, and the range is checked afterwards.  Otherwise the
+  // online form: running maximum m, accumulated output and sum rescaled whenever a maximum moves.
+  auto sweep = [&](auto fast_tag) {
+  constexpr bool FAST = decltype(fast_tag)::value;
+  m = -INFINITY;
+  l = 0.f;
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -209,10 +235,6 @@ window_attention_stream_kernel(StreamParams p) {
     store_chunk(1);
   }
   __syncthreads();
-
-  // A wave whose 32 queries all lie past the window (last query block of a window whose size is not a multiple of 256)
-  // only stages K / V and keeps the barriers; its MFMA and softmax work would be thrown away.
-  const bool wave_active = qb * QB + wave * 32 < L;  // wave-uniform
 
   for (int j = 0; j < nch; ++j) {
     constexpr int LEAD = NBUF / 2;  // chunk j + LEAD is loaded and written to LDS while chunk j is consumed
@@ -269,25 +291,26 @@ window_attention_stream_kernel(StreamParams p) {
     load_v(0, vfb[0]);  // in flight during the softmax arithmetic below
 
     // ---- online softmax (exp2 domain): new row max, rescale what has been accumulated if any max moved
-    float cm = acc[0][0];
+    if (!FAST) {
+      float cm = acc[0][0];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int e = 0; e < 16; e += 2) cm = fmaxf(fmaxf(cm, acc[kb][e]), acc[kb][e + 1]);
-    cm *= c;
-    cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
-    const float m_new = fmaxf(m, cm);
-    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // 0 for the first chunk (m = -inf)
-      l *= alpha;
+        for (int e = 0; e < 16; e += 2) cm = fmaxf(fmaxf(cm, acc[kb][e]), acc[kb][e + 1]);
+      cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+      const float m_new = fmaxf(m, cm);
+      if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // 0 for the first chunk (m = -inf)
+        l *= alpha;
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
-      m = m_new;
+          for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+        m = m_new;
+      }
     }
 
-    // ---- P = exp2(s - m) for 16 keys at a time and O^T += V^T P^T: while the MFMAs of a step run, the P of the next
+    // ---- P = exp2(s) or exp2(s - m) for 16 keys at a time and O^T += V^T P^T: while the MFMAs of a step run, the P of the next
     // step is formed (the VALU work hides the MFMAs) and its V^T fragments are read
     uint32_t pkb[2][4];
     auto exp_step = [&](int step, uint32_t (&pk)[4]) {
@@ -295,8 +318,8 @@ window_attention_stream_kernel(StreamParams p) {
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const int h2 = 4 * t2 + h;
-        const float e0 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2], c, -m));
-        const float e1 = __builtin_amdgcn_exp2f(fmaf(acc[kb][2 * h2 + 1], c, -m));
+        const float e0 = __builtin_amdgcn_exp2f(FAST ? acc[kb][2 * h2] : acc[kb][2 * h2] - m);
+        const float e1 = __builtin_amdgcn_exp2f(FAST ? acc[kb][2 * h2 + 1] : acc[kb][2 * h2 + 1] - m);
         pk[h] = pack_bf16x2(e0, e1);
         l = dot2_ones(pk[h], l);  // the row sum of what PV multiplies: the rounded values, one instruction per pair
       }
@@ -321,6 +344,18 @@ window_attention_stream_kernel(StreamParams p) {
     if (j + LEAD < nch) store_chunk((j + LEAD) & (NBUF - 1));
     if (NBUF == 2 || (j & 1)) __syncthreads();
   }
+  };  // sweep
+
+  sweep(std::true_type{});
+  // Range check of the sweep without maximum: a row sum that left [2^-40, 2^100] (or is not a number) means logits
+  // beyond what exp2 holds without the maximum; the workgroup then repeats the window's keys in the online form.
+  {
+    const float lt = l + __shfl_xor(l, 32, 64);
+    const bool bad = wave_active && !(lt >= 0x1p-40f && lt <= 0x1p100f);
+    if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) *redo = 1;
+    __syncthreads();
+    if (*redo != 0) sweep(std::false_type{});
+  }
 
   // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i]
   l += __shfl_xor(l, 32, 64);
@@ -341,7 +376,7 @@ window_attention_stream_kernel(StreamParams p) {
 
 // ---------------------------------------------------------------------------------------------
 
-static int stream_smem(int head_dim, int L) { return NBUF * (KC * head_dim * 2 + head_dim * KC * 2) + ((L * 4 + 15) / 16) * 16; }
+static int stream_smem(int head_dim, int L) { return NBUF * (KC * head_dim * 2 + head_dim * KC * 2) + ((L * 4 + 15) / 16) * 16 + 16; }
 
 bool attention_stream_supported(int ws_y, int ws_x, int head_dim, bool has_bias, bool use_mask) {
   const int64_t L = (int64_t)ws_y * ws_x;

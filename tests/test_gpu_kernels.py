@@ -240,6 +240,34 @@ def test_window_attention_streaming_parity(pkg, cuda, case):
     assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
 
 
+@pytest.mark.parametrize("case", [
+    # B, H, W, heads, head_dim, ws, q/k magnitude: logits of +-100 and more in the exp2 domain
+    (1, 40, 40, 2, 128, 20, 7.0),
+    (1, 60, 60, 1, 128, 60, 9.0),   # the reference's window
+    (1, 40, 20, 2, 64, 20, 8.0),
+], ids=["ws20_hd128_x7", "ws60_hd128_x9", "ws20_hd64_x8"])
+def test_window_attention_streaming_large_logits(pkg, cuda, case):
+    """The streaming kernel first sweeps the keys without a row maximum and checks the row sums afterwards; logits that
+    overflow exp2 (here: q and k several times larger than N(0,1)) must send the workgroup through the online form and
+    give the same softmax.  Bound as for the one-window kernels at this magnitude: q * scale is rounded to bf16 once
+    more (as in the reference's bf16 path, model.py:290), a few percent of P once logits reach the hundreds."""
+    B, H, W, heads, hd, ws, mag = case
+    g = torch.Generator().manual_seed(int(mag * 10) + hd)
+    inner = heads * hd
+    qkv = torch.randn(B, H * W, 3 * inner, generator=g)
+    qkv[..., :2 * inner] *= mag
+    qkv = bf(qkv)
+    cfg = OracleConfig(dim=inner, heads=heads, head_dim=hd, mlp_dim=inner, window_size=(ws, ws), image_shape=(H, W),
+                       rel_pos_bias=False, shift_mask=False)
+    ref = attention_core(cfg, qkv.float(), (ws // 2, ws // 2), None)
+    out = pkg.ops.window_attention(qkv.to(cuda).view(B * H * W, -1), B, (H, W), heads, hd, (ws, ws), (ws // 2, ws // 2), None, False)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    err = rel_l2(out.view(B, H * W, inner), ref)
+    print(f"streaming attention, |q|,|k| x{mag}: rel-L2 {err:.3e}")
+    assert err <= 3e-2, err
+
+
 HEAD_PLANE_CASES = [
     # B, H, W, heads, hd, ws_y, ws_x, shift, bias, mask -- one-window kernel (small and large grids) and streaming kernel
     (1, 48, 64, 3, 64, 16, 16, 8, True, True),

@@ -68,6 +68,9 @@ struct StreamCfg {
   static constexpr int K_BYTES = KC * HD * 2;
   static constexpr int V_BYTES = HD * KC * 2;
   static constexpr int BUF = K_BYTES + V_BYTES;
+  // the K chunks of all buffers first, then the V^T chunks: with head_dim 128 every K fragment of every buffer is
+  // then within the 64 KB that the offset field of an LDS read reaches from one per-lane base
+  static constexpr int V_BASE = NBUF * K_BYTES;
   static constexpr int TBL_OFF = NBUF * BUF;
 };
 
@@ -177,8 +180,8 @@ window_attention_stream_kernel(StreamParams p) {
     }
   };
   auto store_chunk = [&](int buf) {
-    unsigned char* sK = smem + buf * Cfg::BUF;
-    unsigned char* sV = sK + Cfg::K_BYTES;
+    unsigned char* sK = smem + buf * Cfg::K_BYTES;
+    unsigned char* sV = smem + Cfg::V_BASE + buf * Cfg::V_BYTES;
 #pragma unroll
     for (int it = 0; it < KIT; ++it) {
       const int idx = tid + it * NT, key = idx / CH, c = idx % CH;
@@ -204,12 +207,26 @@ window_attention_stream_kernel(StreamParams p) {
     }
   };
 
-  // head_dim 128: vt_off(32 db + l31, 2 step + hi) = vt_row + 4096 db + vt_x[step ^ db]: the row part and the four possible chunk parts
-  // of this lane (five registers instead of one address per step and row block)
-  const uint32_t vt_row = (uint32_t)((l31 >> 1) * 256 + (l31 & 1) * 128);
-  uint32_t vt_x[4];
+  // Fragment addresses = per-lane part (below, loop-invariant) + compile-time part (buffer, key block / row block):
+  //   K fragment of k16 step s, key block kb:  k_lane[s] + buf * K_BYTES + kb * 32 rows
+  //   V^T fragment of step, row block db:      v_lane[head_dim 128: step ^ db, else step] + V_BASE + buf * V_BYTES + db * 4096
+  // (the swizzles depend on the row only through bits that the block offsets leave alone)
+  // (kept as opaque 32-bit LDS addresses: left to itself the compiler splits them again into a common and a per-step
+  // part and adds the two in front of every read)
+  typedef __attribute__((address_space(3))) const unsigned char* lds_cptr;
+  lds_cptr k_lane[KS], v_lane[4];
 #pragma unroll
-  for (int sx = 0; sx < 4; ++sx) vt_x[sx] = (uint32_t)(((2 * sx) ^ hi ^ ((l31 >> 1) & 7) ^ (l31 >> 4)) << 4);
+  for (int sq = 0; sq < KS; ++sq) {
+    k_lane[sq] = (lds_cptr)(smem + (HD == 64 ? off128(l31, 2 * sq + hi) : off256(l31, 2 * sq + hi)));
+    asm volatile("" : "+v"(k_lane[sq]));
+  }
+#pragma unroll
+  for (int sx = 0; sx < 4; ++sx) {
+    v_lane[sx] = (lds_cptr)(smem + Cfg::V_BASE +
+                 (HD == 128 ? (uint32_t)((l31 >> 1) * 256 + (l31 & 1) * 128) + (uint32_t)(((2 * sx) ^ hi ^ ((l31 >> 1) & 7) ^ (l31 >> 4)) << 4)
+                            : vt_off<HD>(l31, 2 * sx + hi)));
+    asm volatile("" : "+v"(v_lane[sx]));
+  }
   float m = -INFINITY, l = 0.f;
   f32x16 o[DB];
   // A wave whose 32 queries all lie past the window (last query block of a window whose size is not a multiple of 256)
@@ -236,11 +253,14 @@ window_attention_stream_kernel(StreamParams p) {
   }
   __syncthreads();
 
-  for (int j = 0; j < nch; ++j) {
+  // the chunk loop is unrolled over the buffers, so that the buffer a chunk sits in is a compile-time constant
+  for (int j0 = 0; j0 < nch; j0 += NBUF) {
+#pragma unroll
+  for (int u = 0; u < NBUF; ++u) {
+    const int j = j0 + u;
+    if (j >= nch) break;
     constexpr int LEAD = NBUF / 2;  // chunk j + LEAD is loaded and written to LDS while chunk j is consumed
     if (j + LEAD < nch) load_chunk(j + LEAD);
-    const unsigned char* sK = smem + (j & (NBUF - 1)) * Cfg::BUF;
-    const unsigned char* sV = sK + Cfg::K_BYTES;
     f32x16 acc[2];
     if (wave_active) {
 
@@ -254,9 +274,9 @@ window_attention_stream_kernel(StreamParams p) {
     {
       constexpr int PF = 2, NS = 2 * KS;
       bf16x8 kfr[PF + 1];
-      auto read_k = [&](int t) {
-        const int row = (t / KS) * 32 + l31, ch = (t % KS) * 2 + hi;
-        return *reinterpret_cast<const bf16x8*>(sK + (HD == 64 ? off128(row, ch) : off256(row, ch)));
+      auto read_k = [&](int t) {  // rows 32 (t / KS) + l31, 16-byte chunk 2 (t % KS) + hi
+        typedef __attribute__((address_space(3))) const bf16x8* frag_ptr;
+        return *(frag_ptr)(k_lane[t % KS] + u * Cfg::K_BYTES + (t / KS) * 32 * (HD * 2));
       };
 #pragma unroll
       for (int t = 0; t < PF; ++t) kfr[t] = read_k(t);
@@ -283,10 +303,8 @@ window_attention_stream_kernel(StreamParams p) {
     bf16x8 vfb[2][DB];
     auto load_v = [&](int step, bf16x8 (&f)[DB]) {  // f[db] = V^T rows 32 db + l31, chunk step * 2 + hi: vt_off(), taken apart
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        if (HD == 128) f[db] = *reinterpret_cast<const bf16x8*>(sV + vt_row + db * 4096 + vt_x[step ^ db]);
-        else f[db] = *reinterpret_cast<const bf16x8*>(sV + vt_off<HD>(db * 32 + l31, step * 2 + hi));
-      }
+      for (int db = 0; db < DB; ++db)
+        f[db] = *(__attribute__((address_space(3))) const bf16x8*)(v_lane[HD == 128 ? step ^ db : step] + u * Cfg::V_BYTES + db * 4096);
     };
     load_v(0, vfb[0]);  // in flight during the softmax arithmetic below
 
@@ -341,8 +359,9 @@ window_attention_stream_kernel(StreamParams p) {
     __builtin_amdgcn_sched_barrier(0);
     }  // wave_active
 
-    if (j + LEAD < nch) store_chunk((j + LEAD) & (NBUF - 1));
-    if (NBUF == 2 || (j & 1)) __syncthreads();
+    if (j + LEAD < nch) store_chunk((u + LEAD) & (NBUF - 1));
+    if (NBUF == 2 || (u & 1)) __syncthreads();
+  }
   }
   };  // sweep
 

@@ -35,6 +35,7 @@ struct StreamParams {
   int sy, sx;
   int n_units, qblks;
   float scale;
+  uint32_t span_bytes;  // DMA form: bytes of one image's k (or v) plane that a token offset can reach, < 2^32
 };
 
 constexpr int KC = 64;    // keys per chunk
@@ -76,9 +77,17 @@ struct StreamCfg {
 
 }  // namespace
 
-template <int HD>
+// DMA (head_dim 128): K and V chunks go into LDS by the load unit itself (buffer_load ... lds: no staging registers,
+// no ds_write, no transposing VALU work) and V stays row-major; the V^T fragments of P V then come from
+// ds_read_b64_tr_b16, the LDS read that transposes on the way out (within 16 lanes, source lane 4e + a reads 4
+// consecutive elements and result lane 4a + b receives element b of source lanes a, 4 + a, 8 + a, 12 + a).  Rows of
+// 256 B, 16-byte chunks XOR-swizzled: K by row & 15 (conflict-free ds_read_b128 fragments), V by 2 (row & 3) (the 4
+// keys x 4 column groups one transposing read gathers per 16 lanes hit distinct banks).  Needs every byte offset
+// inside an image's k / v plane to fit 32 bits (span_bytes; checked by the launcher).
+template <int HD, bool DMA>
 __global__ void __launch_bounds__(64 * NWAVE) __attribute__((amdgpu_waves_per_eu(2)))
 window_attention_stream_kernel(StreamParams p) {
+  static_assert(!DMA || HD == 128, "the DMA form is built for head_dim 128");
   using Cfg = StreamCfg<HD>;
   constexpr int CH = HD / 8;   // 16-byte chunks per head row
   constexpr int KS = HD / 16;  // k16 steps of QK^T
@@ -207,6 +216,39 @@ window_attention_stream_kernel(StreamParams p) {
     }
   };
 
+  // DMA form: one instruction of a wave fills 1 KB = 4 rows of a chunk; wave w issues rows 4w.. and 32 + 4w.. of K and
+  // of V.  Lane = (row within the four, LDS chunk slot); it fetches the global chunk that the swizzle keeps there.
+  // Keys past the window get an offset outside the descriptor and arrive as zeros (their scores are masked).
+  typedef __attribute__((address_space(3))) void* lds_vptr;
+  const __amdgpu_buffer_rsrc_t rs_k = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)p.span_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_v = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (int)p.span_bytes, 0x00020000);
+  auto issue_chunk = [&](int j, int buf) {
+    const int rsub = lane >> 4, pc = lane & 15;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int ii = wave + NWAVE * i;  // 0..15
+      const int row = 4 * ii + rsub, key = j * KC + row;
+      const uint32_t rowoff = key < L ? (uint32_t)tok[key < L ? key : 0] * (ld_qkv * 2u) : 0xFFFFF000u;
+      const uint32_t ok = rowoff + (uint32_t)((pc ^ (row & 15)) << 4), ov = rowoff + (uint32_t)((pc ^ (2 * rsub)) << 4);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_k, (lds_vptr)(smem + buf * Cfg::K_BYTES + ii * 1024), 16, ok, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_v, (lds_vptr)(smem + Cfg::V_BASE + buf * Cfg::V_BYTES + ii * 1024), 16, ov, 0, 0, 0);
+    }
+  };
+  // per-lane part of the transposing V reads: block of 16 lanes jb = lane >> 4 (d half jb & 1, key half jb >> 1),
+  // source lane 4e + a inside it reads V[key0 + 4 (jb >> 1) + e][32 db + 16 (jb & 1) + 4a ..]
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr;
+  uint32_t v_tr[DB];
+  if (DMA) {
+    const int jb = lane >> 4, e = (lane >> 2) & 3, a = lane & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = (4 * db + 2 * (jb & 1) + (a >> 1)) ^ (2 * e);
+      v_tr[db] = (uint32_t)(Cfg::V_BASE + (4 * (jb >> 1) + e) * (HD * 2) + (chunk << 4) + (a & 1) * 8);
+      asm volatile("" : "+v"(v_tr[db]));
+    }
+  }
+
   // Fragment addresses = per-lane part (below, loop-invariant) + compile-time part (buffer, key block / row block):
   //   K fragment of k16 step s, key block kb:  k_lane[s] + buf * K_BYTES + kb * 32 rows
   //   V^T fragment of step, row block db:      v_lane[head_dim 128: step ^ db, else step] + V_BASE + buf * V_BYTES + db * 4096
@@ -245,11 +287,17 @@ window_attention_stream_kernel(StreamParams p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
 
-  load_chunk(0);
-  store_chunk(0);
-  if (NBUF == 4 && nch > 1) {
-    load_chunk(1);
-    store_chunk(1);
+  if (DMA) {
+    issue_chunk(0, 0);
+    if (nch > 1) issue_chunk(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): this wave's loads into LDS have landed
+  } else {
+    load_chunk(0);
+    store_chunk(0);
+    if (NBUF == 4 && nch > 1) {
+      load_chunk(1);
+      store_chunk(1);
+    }
   }
   __syncthreads();
 
@@ -260,7 +308,16 @@ window_attention_stream_kernel(StreamParams p) {
     const int j = j0 + u;
     if (j >= nch) break;
     constexpr int LEAD = NBUF / 2;  // chunk j + LEAD is loaded and written to LDS while chunk j is consumed
-    if (j + LEAD < nch) load_chunk(j + LEAD);
+    if (DMA) {
+      // both chunks of the next pair are requested at the start of this pair (the buffers were last read before the
+      // barrier that ended the pair before), and awaited at the barrier that ends this pair
+      if ((u & 1) == 0) {
+        if (j + LEAD < nch) issue_chunk(j + LEAD, (u + LEAD) & (NBUF - 1));
+        if (j + LEAD + 1 < nch) issue_chunk(j + LEAD + 1, (u + LEAD + 1) & (NBUF - 1));
+      }
+    } else if (j + LEAD < nch) {
+      load_chunk(j + LEAD);
+    }
     f32x16 acc[2];
     if (wave_active) {
 
@@ -303,8 +360,16 @@ window_attention_stream_kernel(StreamParams p) {
     bf16x8 vfb[2][DB];
     auto load_v = [&](int step, bf16x8 (&f)[DB]) {  // f[db] = V^T rows 32 db + l31, chunk step * 2 + hi: vt_off(), taken apart
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-        f[db] = *(__attribute__((address_space(3))) const bf16x8*)(v_lane[HD == 128 ? step ^ db : step] + u * Cfg::V_BYTES + db * 4096);
+      for (int db = 0; db < DB; ++db) {
+        if (DMA) {  // keys 16 step + 4 hi + (0..3) and 16 step + 8 + 4 hi + (0..3) of row-major V, transposed by the read
+          const uint32_t a0 = v_tr[db] + u * Cfg::V_BYTES + step * 16 * (HD * 2);
+          const bf16x4_t lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(smem + a0));
+          const bf16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(smem + a0 + 8 * (HD * 2)));
+          f[db] = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+          f[db] = *(__attribute__((address_space(3))) const bf16x8*)(v_lane[HD == 128 ? step ^ db : step] + u * Cfg::V_BYTES + db * 4096);
+        }
+      }
     };
     load_v(0, vfb[0]);  // in flight during the softmax arithmetic below
 
@@ -359,8 +424,11 @@ window_attention_stream_kernel(StreamParams p) {
     __builtin_amdgcn_sched_barrier(0);
     }  // wave_active
 
-    if (j + LEAD < nch) store_chunk((u + LEAD) & (NBUF - 1));
-    if (NBUF == 2 || (u & 1)) __syncthreads();
+    if (!DMA && j + LEAD < nch) store_chunk((u + LEAD) & (NBUF - 1));
+    if (NBUF == 2 || (u & 1)) {
+      if (DMA) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the next pair's chunks, requested two chunks ago
+      __syncthreads();
+    }
   }
   }
   };  // sweep
@@ -403,10 +471,13 @@ bool attention_stream_supported(int ws_y, int ws_x, int head_dim, bool has_bias,
 }
 
 hipError_t attention_stream_configure_all() {
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_stream_kernel<64>),
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_stream_kernel<64, false>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, stream_smem(64, MAX_L));
   if (e != hipSuccess) return e;
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_stream_kernel<128>),
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_stream_kernel<128, false>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, stream_smem(128, MAX_L));
+  if (e != hipSuccess) return e;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_stream_kernel<128, true>),
                              hipFuncAttributeMaxDynamicSharedMemorySize, stream_smem(128, MAX_L));
 }
 
@@ -426,10 +497,15 @@ hipError_t attention_stream_launch(const void* qkv, void* out, int B, int H, int
   p.qblks = (L + QB - 1) / QB;
   const int64_t grid = (int64_t)((p.n_units + 7) / 8) * 8 * p.qblks;
   const int smem = stream_smem(head_dim, L);
+  // bytes of an image's k (or v) plane that a token offset can reach; the DMA form addresses them with 32 bits
+  const int64_t span = ((int64_t)H * W - 1) * tok_stride * 2 + (int64_t)head_dim * 2;
+  p.span_bytes = span < ((int64_t)1 << 32) - 4096 ? (uint32_t)span : 0u;
   if (head_dim == 64)
-    hipLaunchKernelGGL(window_attention_stream_kernel<64>, dim3((unsigned)grid), dim3(64 * NWAVE), smem, stream, p);
+    hipLaunchKernelGGL((window_attention_stream_kernel<64, false>), dim3((unsigned)grid), dim3(64 * NWAVE), smem, stream, p);
+  else if (p.span_bytes != 0 && tok_stride > 0)
+    hipLaunchKernelGGL((window_attention_stream_kernel<128, true>), dim3((unsigned)grid), dim3(64 * NWAVE), smem, stream, p);
   else
-    hipLaunchKernelGGL(window_attention_stream_kernel<128>, dim3((unsigned)grid), dim3(64 * NWAVE), smem, stream, p);
+    hipLaunchKernelGGL((window_attention_stream_kernel<128, false>), dim3((unsigned)grid), dim3(64 * NWAVE), smem, stream, p);
   return hipGetLastError();
 }
 

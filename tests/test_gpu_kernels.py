@@ -268,6 +268,30 @@ def test_window_attention_streaming_large_logits(pkg, cuda, case):
     assert err <= 3e-2, err
 
 
+def test_window_attention_streaming_wide_rows_match_compact(pkg, cuda):
+    """head_dim 128 has two streaming forms: K / V straight into LDS by the load unit when every token offset of an
+    image's k / v plane fits 32 bits, through registers otherwise.  A [S, 3 * inner] matrix with 388 heads (token
+    stride 298 KB, 4.3 GB in all) takes the second; a compact copy of three of its heads takes the first.  Same
+    arithmetic in the same order: the outputs must agree bit for bit."""
+    H = W = 120
+    heads, hd, ws = 388, 128, 60
+    S, inner = H * W, heads * hd
+    g = torch.Generator(device=cuda).manual_seed(11)
+    qkv = torch.empty(S, 3 * inner, dtype=torch.bfloat16, device=cuda)
+    for c0 in range(0, 3 * inner, 16384):  # filled in slabs: no 17 GB f32 temporary
+        c1 = min(c0 + 16384, 3 * inner)
+        qkv[:, c0:c1] = torch.randn(S, c1 - c0, generator=g, device=cuda).to(torch.bfloat16)
+    out = pkg.ops.window_attention(qkv, 1, (H, W), heads, hd, (ws, ws), (30, 30), None, False)
+    pick = [0, 201, 387]
+    cols = torch.cat([torch.arange(c * inner + h * hd, c * inner + (h + 1) * hd) for c in range(3) for h in pick]).to(cuda)
+    small = qkv.index_select(1, cols).contiguous()  # [S, 3 * 3 * 128], columns ordered (c h d) like the big one
+    out_small = pkg.ops.window_attention(small, 1, (H, W), len(pick), hd, (ws, ws), (30, 30), None, False)
+    torch.cuda.synchronize()
+    for i, h in enumerate(pick):
+        assert torch.equal(out[:, h * hd:(h + 1) * hd], out_small[:, i * hd:(i + 1) * hd]), h
+    assert bool(torch.isfinite(out_small.float()).all()) and float(out_small.float().abs().mean()) > 1e-3
+
+
 HEAD_PLANE_CASES = [
     # B, H, W, heads, hd, ws_y, ws_x, shift, bias, mask -- one-window kernel (small and large grids) and streaming kernel
     (1, 48, 64, 3, 64, 16, 16, 8, True, True),

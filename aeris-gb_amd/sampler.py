@@ -65,6 +65,7 @@ class _Rollout:
             self.latents = latents.to(dev, torch.float32).contiguous()
         self.B = B
         self.graph, self.step = None, None
+        self.steps_per_replay = 1  # forecast steps recorded in ``graph``
         self._done = 0
         self.reset()
 
@@ -80,11 +81,14 @@ class _Rollout:
         n = self.n_forecast - self._done if n is None else n
         if n < 0 or self._done + n > self.n_forecast:
             raise ValueError(f"{self._done} of {self.n_forecast} forecast steps are done; cannot run {n} more (reset() first)")
+        if self.graph is not None and n % self.steps_per_replay:
+            raise ValueError(f"the captured graph holds {self.steps_per_replay} forecast steps; {n} is not a multiple of that")
         self._done += n
-        for _ in range(n):
-            if self.graph is not None:
+        if self.graph is not None:
+            for _ in range(n // self.steps_per_replay):
                 self.graph.replay()
-            else:
+        else:
+            for _ in range(n):
                 self.step()
         return self.states
 
@@ -186,12 +190,17 @@ class TrigFlowSampler:
     @torch.no_grad()
     def begin_rollout(self, state0: torch.Tensor, n_forecast: int, generator: Optional[torch.Generator] = None,
                       x_mean=None, x_std=None, t_mean=None, t_std=None, forcing=None, static=None, extra_cond=None,
-                      latents=None, use_graph=False, graph_warmup: int = 0) -> "_Rollout":
-        """Set up an autoregressive forecast (arguments: see ``rollout``) and, with ``use_graph``, capture its
-        forecast step (after ``graph_warmup`` eager steps, whose effect on the state is undone).  ``run()`` of the
-        returned object advances it; ``reset()`` puts it back to ``state0`` and step 0."""
+                      latents=None, use_graph=False, graph_warmup: int = 0, graph_steps: int = 1) -> "_Rollout":
+        """Set up an autoregressive forecast (arguments: see ``rollout``) and, with ``use_graph``, capture
+        ``graph_steps`` consecutive forecast steps as one HIP graph (1: the graph is one forecast step and is replayed
+        per step; n_forecast: the whole rollout is one graph and one replay), after ``graph_warmup`` eager steps whose
+        effect on the state is undone.  The forecast-step counter, the forcings and the state store are indexed on the
+        device, so the same recorded step serves every position of the rollout.  ``run()`` of the returned object
+        advances it; ``reset()`` puts it back to ``state0`` and step 0."""
         if not 0 <= graph_warmup <= n_forecast:
             raise ValueError(f"graph_warmup must lie in 0..{n_forecast} (the warm-up steps are forecast steps)")
+        if graph_steps < 1 or n_forecast % graph_steps:
+            raise ValueError(f"graph_steps must divide n_forecast = {n_forecast}")
         ro = _Rollout(state0, n_forecast, x_mean, x_std, t_mean, t_std, forcing, static, extra_cond, latents)
         if use_graph and generator is None and latents is None:
             generator = torch.cuda.default_generators[state0.device.index or 0]
@@ -200,7 +209,20 @@ class TrigFlowSampler:
         if use_graph:
             # the default generator is registered with every graph; any other one has to be registered by hand
             own = gen if gen is not None and gen is not torch.cuda.default_generators[state0.device.index or 0] else None
-            ro.graph = self._capture(ro.step, graph_warmup, generator=own)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(graph_warmup):
+                    ro.step()
+            torch.cuda.current_stream().wait_stream(side)
+            ro.reset()
+
+            def steps():
+                for _ in range(graph_steps):
+                    ro.step()
+
+            ro.steps_per_replay = graph_steps
+            ro.graph = self._capture(steps if graph_steps > 1 else ro.step, 0, generator=own)
             ro.reset()
         return ro
 
@@ -213,7 +235,8 @@ class TrigFlowSampler:
         ``state0`` is the standardised state [B, S, C]; ``x_mean, x_std, t_mean, t_std`` are per-channel tensors [C]
         (identity when omitted); ``forcing`` [n_forecast + 1, 1|B, S, Cf]; ``static`` [1|B, S, Cs]; ``extra_cond``
         [1|B, S, Ce] or one per step [n_forecast, 1|B, S, Ce]; ``latents`` [n_forecast, B, S, C] replaces the draw
-        from ``generator``.  ``use_graph``: the forecast step is captured once and replayed n_forecast times.
+        from ``generator``.  ``use_graph``: the forecast step is captured once and replayed n_forecast times
+        (``graph_steps=n_forecast``: the whole rollout is captured as one graph and replayed once).
         Returns the standardised state after every forecast step, [n_forecast, B, S, C].
         """
         ro = self.begin_rollout(state0, n_forecast, generator, **kw)

@@ -202,6 +202,15 @@ def test_rollout_parity_eager_and_graph(pkg, cuda):
         model(torch.randn(B, S, cfg.in_channels, device=cuda), torch.tensor([0.3], device=cuda))
         torch.cuda.synchronize()
         assert torch.equal(ro.states[k], eager[k]), k
+    # the whole rollout as ONE graph and one replay (the step counter, forcings and state store are indexed on the device)
+    whole = smp.begin_rollout(state0.to(cuda), n_fc, use_graph=True, graph_steps=n_fc, **dkw)
+    assert torch.equal(whole.run(), eager)
+    whole.reset()
+    model(torch.randn(B, S, cfg.in_channels, device=cuda), torch.tensor([0.7], device=cuda))  # eager work in between
+    assert torch.equal(whole.run(), eager)
+    with pytest.raises(ValueError, match="multiple"):
+        whole.reset()
+        whole.run(1)
     # a generator instead of given latents: the graph draws its latents on the device, every replay new ones
     gen = torch.Generator(device="cuda").manual_seed(3)
     drawn = smp.rollout(state0.to(cuda), 2, gen, use_graph=True, **{k: v for k, v in dkw.items() if k != "latents"})

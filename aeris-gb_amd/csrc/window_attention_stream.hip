@@ -81,8 +81,9 @@ struct StreamCfg {
 // no ds_write, no transposing VALU work) and V stays row-major; the V^T fragments of P V then come from
 // ds_read_b64_tr_b16, the LDS read that transposes on the way out (within 16 lanes, source lane 4e + a reads 4
 // consecutive elements and result lane 4a + b receives element b of source lanes a, 4 + a, 8 + a, 12 + a).  Rows of
-// 256 B, 16-byte chunks XOR-swizzled: K by row & 15 (conflict-free ds_read_b128 fragments), V by 2 (row & 3) (the 4
-// keys x 4 column groups one transposing read gathers per 16 lanes hit distinct banks).  Needs every byte offset
+// 256 B, 16-byte chunks XOR-swizzled: K by row & 15 (conflict-free ds_read_b128 fragments), V by 4 (row & 3) (the 4
+// keys x 4 column groups that the two 16-lane halves of a transposing read's 32-lane pass gather - 16 pieces of 16
+// bytes - land on the 16 distinct slots of a 256-byte bank period; with 2 (row & 3) the two halves shared eight).  Needs every byte offset
 // inside an image's k / v plane to fit 32 bits (span_bytes; checked by the launcher).
 template <int HD, bool DMA>
 __global__ void __launch_bounds__(64 * NWAVE) __attribute__((amdgpu_waves_per_eu(2)))
@@ -229,7 +230,7 @@ window_attention_stream_kernel(StreamParams p) {
       const int ii = wave + NWAVE * i;  // 0..15
       const int row = 4 * ii + rsub, key = j * KC + row;
       const uint32_t rowoff = key < L ? (uint32_t)tok[key < L ? key : 0] * (ld_qkv * 2u) : 0xFFFFF000u;
-      const uint32_t ok = rowoff + (uint32_t)((pc ^ (row & 15)) << 4), ov = rowoff + (uint32_t)((pc ^ (2 * rsub)) << 4);
+      const uint32_t ok = rowoff + (uint32_t)((pc ^ (row & 15)) << 4), ov = rowoff + (uint32_t)((pc ^ (4 * rsub)) << 4);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_k, (lds_vptr)(smem + buf * Cfg::K_BYTES + ii * 1024), 16, ok, 0, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_v, (lds_vptr)(smem + Cfg::V_BASE + buf * Cfg::V_BYTES + ii * 1024), 16, ov, 0, 0, 0);
     }
@@ -243,7 +244,7 @@ window_attention_stream_kernel(StreamParams p) {
     const int jb = lane >> 4, e = (lane >> 2) & 3, a = lane & 3;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      const int chunk = (4 * db + 2 * (jb & 1) + (a >> 1)) ^ (2 * e);
+      const int chunk = (4 * db + 2 * (jb & 1) + (a >> 1)) ^ (4 * e);
       v_tr[db] = (uint32_t)(Cfg::V_BASE + (4 * (jb >> 1) + e) * (HD * 2) + (chunk << 4) + (a & 1) * 8);
       asm volatile("" : "+v"(v_tr[db]));
     }

@@ -4,7 +4,7 @@ The grid is the only thing that is reduced (the oracle has to finish in seconds)
 length, head count, window size and weight shapes of the benchmarked step, and the residual stream passes
 through all 24 blocks.  After every block the hidden state is compared (relative L2 and max-abs), which gives the
 error-growth curve; the final output has to be within the benchmark's tolerance of 1e-2 relative L2.
-The curves are printed and, where the directory can be written, stored as JSON under gpurun_out/.
+The curves are printed and, where the directory can be written, stored as JSON in the run's output directory.
 """
 import json
 import os

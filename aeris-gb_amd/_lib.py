@@ -30,7 +30,7 @@ SIGNATURES = {
     "aeris_relative_position_index": (_c_int, [_c_int, _c_int, _c_vp]),
     "aeris_shift_region_ids": (_c_int, [_c_int] * 6 + [_c_vp]),
     "aeris_window_attention_fwd": (_c_int, [_c_vp, _c_vp, _c_vp] + [_c_int] * 10 + [_c_f32, _c_vp]),
-    "aeris_window_attention_heads_fwd": (_c_int, [_c_vp, _c_vp, _c_vp] + [_c_int] * 10 + [_c_f32, _c_i64, _c_vp]),
+    "aeris_window_attention_heads_fwd": (_c_int, [_c_vp, _c_vp, _c_vp] + [_c_int] * 10 + [_c_f32, _c_int, _c_i64, _c_vp]),
     "aeris_norm_modulate_fwd": (_c_int, [_c_vp, _c_int, _c_vp, _c_int, _c_vp, _c_vp, _c_int, _c_vp, _c_vp, _c_i64, _c_i64,
                                          _c_i64, _c_int, _c_int, _c_int, _c_f32, _c_vp]),
     "aeris_output_stage_workspace_bytes": (_c_i64, [_c_int, _c_int, _c_int]),
@@ -40,7 +40,8 @@ SIGNATURES = {
                                                 _c_i64, _c_int, _c_int, _c_int, _c_f32, _c_vp]),
     "aeris_gemm_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_i64, _c_int,
                                 _c_int, _c_int, _c_i64, _c_i64, _c_vp]),
-    "aeris_gemm_heads_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_int, _c_i64, _c_vp]),
+    "aeris_gemm_heads_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_int, _c_i64, _c_f32, _c_int,
+                                      _c_vp]),
     "aeris_modulation_linear_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_vp]),
     "aeris_timestep_embedding_fwd": (_c_int, [_c_vp, _c_vp, _c_int, _c_int, _c_f32, _c_vp]),
     "aeris_embed_prepare_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_vp]),

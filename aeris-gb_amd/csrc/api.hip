@@ -134,7 +134,8 @@ int aeris_shift_region_ids(int H, int W, int ws_y, int ws_x, int shift_y, int sh
 
 static int window_attention_impl(const char* who, const void* qkv, void* out, const void* bias_table, int B, int H, int W,
                                  int heads, int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask,
-                                 float scale, int64_t tok_stride, int64_t head_stride, int64_t part_stride, void* stream) {
+                                 float scale, int q_prescaled, int64_t tok_stride, int64_t head_stride, int64_t part_stride,
+                                 void* stream) {
   if (!qkv || !out) return fail(AERIS_EINVAL, "%s: qkv/out is NULL", who);
   if (!aligned16(qkv) || !aligned16(out)) return fail(AERIS_EINVAL, "%s: qkv/out must be 16-byte aligned", who);
   if (heads <= 0 || head_dim <= 0) return fail(AERIS_EINVAL, "%s: heads/head_dim must be positive", who);
@@ -155,12 +156,13 @@ static int window_attention_impl(const char* who, const void* qkv, void* out, co
   if (int rc = ensure_init(stream, true)) return rc;
   if (!small) {
     hipError_t e = aeris::attention_stream_launch(qkv, out, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x, scale,
-                                                  tok_stride, head_stride, part_stride, reinterpret_cast<hipStream_t>(stream));
+                                                  q_prescaled, tok_stride, head_stride, part_stride,
+                                                  reinterpret_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "window attention launch (streaming kernel)");
     return AERIS_OK;
   }
   hipError_t e = aeris::attention_launch(qkv, out, bias_table, B, H, W, heads, head_dim, ws_y, ws_x, shift_y, shift_x,
-                                         use_mask, scale, tok_stride, head_stride, part_stride,
+                                         use_mask, scale, q_prescaled, tok_stride, head_stride, part_stride,
                                          reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "window attention launch");
   return AERIS_OK;
@@ -171,17 +173,17 @@ int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_tabl
                                void* stream) {
   const int64_t inner = (int64_t)heads * head_dim;
   return window_attention_impl("aeris_window_attention_fwd", qkv, out, bias_table, B, H, W, heads, head_dim, ws_y, ws_x,
-                               shift_y, shift_x, use_mask, scale, 3 * inner, head_dim, inner, stream);
+                               shift_y, shift_x, use_mask, scale, 0, 3 * inner, head_dim, inner, stream);
 }
 
 int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const void* bias_table, int B, int H, int W, int heads,
                                      int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
-                                     int64_t plane_stride, void* stream) {
+                                     int q_prescaled, int64_t plane_stride, void* stream) {
   if (head_dim > 0 && B > 0 && H > 0 && W > 0 && (plane_stride < (int64_t)B * H * W * head_dim || plane_stride % 8))
     return fail(AERIS_EINVAL, "aeris_window_attention_heads_fwd: plane_stride must be a multiple of 8 and at least B*H*W*head_dim");
   return window_attention_impl("aeris_window_attention_heads_fwd", qkv_planes, out, bias_table, B, H, W, heads, head_dim, ws_y,
-                               ws_x, shift_y, shift_x, use_mask, scale, head_dim, plane_stride, (int64_t)heads * plane_stride,
-                               stream);
+                               ws_x, shift_y, shift_x, use_mask, scale, q_prescaled ? 1 : 0, head_dim, plane_stride,
+                               (int64_t)heads * plane_stride, stream);
 }
 
 int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,
@@ -307,13 +309,13 @@ int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, cons
   if ((int64_t)((M + 127) / 128) * ((N + 63) / 64) > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_fwd: too many tiles");
   if (int rc = ensure_init(stream, true)) return rc;
   hipError_t e = aeris::gemm_launch(A, W, C, bias, gate, residual, M, N, K, ldc, act, res_dtype, c_dtype,
-                                    gate_batch_stride, rows_per_batch, 0, 0, reinterpret_cast<hipStream_t>(stream));
+                                    gate_batch_stride, rows_per_batch, 0, 0, 1.0f, 0, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_gemm_fwd launch");
   return AERIS_OK;
 }
 
 int aeris_gemm_heads_fwd(const void* A, const void* W, void* C, const void* bias, int64_t M, int N, int K, int head_dim,
-                         int64_t plane_stride, void* stream) {
+                         int64_t plane_stride, float q_scale, int q_planes, void* stream) {
   if (!A || !W || !C) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: A/W/C is NULL");
   if (M <= 0 || N <= 0 || K <= 0) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: M, N, K must be positive");
   if (!aligned16(A) || !aligned16(W) || !aligned16(C)) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: A/W/C must be 16-byte aligned");
@@ -323,9 +325,13 @@ int aeris_gemm_heads_fwd(const void* A, const void* W, void* C, const void* bias
   if (plane_stride < M * head_dim || plane_stride % 8)
     return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: plane_stride must be a multiple of 8 and at least M * head_dim");
   if ((int64_t)((M + 127) / 128) * ((N + 63) / 64) > 0x7fffffffLL) return fail(AERIS_EUNSUPPORTED, "aeris_gemm_heads_fwd: too many tiles");
+  if (q_planes < 0 || (int64_t)q_planes * head_dim > N)
+    return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: q_planes=%d must lie in [0, N / head_dim]", q_planes);
+  if (q_planes > 0 && !(q_scale > 0.f && q_scale < 3.0e38f)) return fail(AERIS_EINVAL, "aeris_gemm_heads_fwd: q_scale must be positive and finite");
   if (int rc = ensure_init(stream, true)) return rc;
   hipError_t e = aeris::gemm_launch(A, W, C, bias, nullptr, nullptr, M, N, K, N, AERIS_ACT_NONE, -1, AERIS_BF16, 0, M, head_dim,
-                                    plane_stride, reinterpret_cast<hipStream_t>(stream));
+                                    plane_stride, q_planes > 0 ? q_scale : 1.0f, q_planes * head_dim,
+                                    reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "aeris_gemm_heads_fwd launch");
   return AERIS_OK;
 }

@@ -184,6 +184,7 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_nt_kernel(GemmParams p)
             else if (p.act == AERIS_ACT_SILU) x = silu_f(x);
           }
           if (gate_row) x *= gate_row[nn];
+          if (nn < p.q_cols) x *= p.q_scale;
           v[e] = x;
         }
         const int64_t off = m * c_row_stride(p) + c_col_off(p, n);
@@ -253,8 +254,10 @@ hipError_t gemm_configure_all() {
 hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, const float* gate,
                        const void* residual, int64_t M, int N, int K, int64_t ldc, int act, int res_dtype,
                        int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, int split, int64_t plane_stride,
-                       hipStream_t stream) {
+                       float q_scale, int q_cols, hipStream_t stream) {
   GemmParams p;
+  p.q_scale = q_scale;
+  p.q_cols = q_cols;
   p.split = split;
   p.plane_stride = plane_stride;
   p.A = reinterpret_cast<const uint16_t*>(A);
@@ -285,7 +288,9 @@ hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, 
   const bool dma_ok = (int64_t)(swiglu ? 2 : 1) * N * K * 2 < (int64_t(1) << 31) && (K % 64) == 0 && ldc < (1 << 23) && split < (1 << 23) &&
                       gate_batch_stride < (int64_t(1) << 31) && (rows_per_batch <= 0 || M / rows_per_batch < (int64_t(1) << 31)) &&
                       ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15) == 0;
-  if (big && dma_ok && act != AERIS_ACT_SILU && (gate_batch_stride & 3) == 0 && aligned) return gemm_persistent_launch(p, stream);
+  // (the persistent kernel scales whole 64-column wave blocks of the query part)
+  if (big && dma_ok && act != AERIS_ACT_SILU && (gate_batch_stride & 3) == 0 && aligned && q_cols % 64 == 0)
+    return gemm_persistent_launch(p, stream);
   return swiglu ? launch_gemm<128, 128, 2, 2, true, true>(p, stream) : launch_gemm<128, 128, 2, 2, false, true>(p, stream);
 }
 

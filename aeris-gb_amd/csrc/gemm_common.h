@@ -30,6 +30,11 @@ struct GemmParams {
   int act;
   int res_dtype;  // -1 none, AERIS_BF16, AERIS_F32
   int c_dtype;
+  // output columns n < q_cols are multiplied by q_scale in fp32, after the bias and before the only rounding (the
+  // query part of a qkv projection: softmax scale times log2(e)); q_cols = 0: none.  bf16 C without activation,
+  // gate and residual only.
+  float q_scale;
+  int q_cols;
 };
 
 // offset of the group of columns starting at n (a group never straddles a column block) within its row, and the

@@ -232,6 +232,16 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     const int rrow_t = rrow;
     const int n_wave = tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
     u32x2 bq_next[FN];  // loaded ahead of the last block's stores, used after them
+    // The query part of a qkv projection is multiplied by q_scale here, in fp32, before its only rounding.  Whole
+    // 64-column wave blocks lie inside or outside the query columns (q_cols % 64 == 0, checked at launch): a
+    // wave-uniform branch that two thirds of the tiles of such a projection skip.
+    if (PLAIN && ACT == AERIS_ACT_NONE && !OUT_F32 && n_wave < p.q_cols) {
+      const float qs = p.q_scale;
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] *= qs;
+    }
     // Staging area of this wave, 32 rows of 128 B: the A stage that the loader fills next is idle during the
     // epilogue, and the 4 KB of it that this wave's own loads will fill are written by nobody else.
     unsigned char* stg = smem + la_stage * A_BYTES + wave_u * 4096;

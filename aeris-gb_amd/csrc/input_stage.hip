@@ -116,7 +116,7 @@ __global__ void __launch_bounds__(IS_THREADS, 2) input_stage_kernel(InStageParam
   const int x1_stride = p.x1 ? p.C1 : C0;
   const float* const apeb = p.ape ? p.ape : p.x0;
   const int ape_stride = p.ape ? C : 0, ape_kmask = p.ape ? -1 : 0;
-  const float has_ape = p.ape ? 1.0f : 0.0f;
+  const bool has_ape = p.ape != nullptr;  // wave-uniform
   const float inv_div = 1.0f / p.div0;
 #pragma unroll
   for (int rb = 0; rb < IS_RB; ++rb) {
@@ -148,7 +148,10 @@ __global__ void __launch_bounds__(IS_THREADS, 2) input_stage_kernel(InStageParam
           // x / div0 for the state channels: quotient by reciprocal with one correction step
           float quo = x * inv_div;
           quo = fmaf(fmaf(-quo, p.div0, x), inv_div, quo);
-          const float v = fmaf(a, has_ape, first ? quo : x);
+          // without a positional encoding `a` is a stand-in read from the input itself: a select, not a multiply
+          // by zero, keeps an Inf or NaN there out of every other token
+          const float base = first ? quo : x;
+          const float v = has_ape ? a + base : base;
           val[rr][g] = k < C ? v : (k == C ? 1.0f : 0.0f);
         }
       }
@@ -214,6 +217,7 @@ __global__ void __launch_bounds__(IS_THREADS, 2) input_stage_kernel(InStageParam
     }
     // The DMA loads of the next chunk were issued ahead of this chunk's 16 stores and vector memory operations
     // complete in order: "all but the newest 16" is exactly those loads, without waiting for any store.
+    static_assert(IS_NBC * IS_RB == 16, "the vmcnt(16) below counts one store per 16-column block and 16-row block");
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16)
     __builtin_amdgcn_s_barrier();

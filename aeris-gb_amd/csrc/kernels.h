@@ -13,7 +13,7 @@ hipError_t attention_configure_all();
 hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, const float* gate,
                        const void* residual, int64_t M, int N, int K, int64_t ldc, int act, int res_dtype,
                        int c_dtype, int64_t gate_batch_stride, int64_t rows_per_batch, int split, int64_t plane_stride,
-                       hipStream_t stream);
+                       float q_scale, int q_cols, hipStream_t stream);
 
 // returns hipErrorInvalidValue when (ws_y, ws_x, head_dim) has no instantiation.  q / k / v of (token, head) start at
 // part * part_stride + head * head_stride + token * tok_stride (elements) for part = 0, 1, 2
@@ -22,11 +22,12 @@ bool attention_supported(int ws_y, int ws_x, int head_dim);
 bool attention_stream_supported(int ws_y, int ws_x, int head_dim, bool has_bias, bool use_mask);
 hipError_t attention_stream_configure_all();
 hipError_t attention_stream_launch(const void* qkv, void* out, int B, int H, int W, int heads, int head_dim, int ws_y,
-                                   int ws_x, int shift_y, int shift_x, float scale, int64_t tok_stride, int64_t head_stride,
-                                   int64_t part_stride, hipStream_t stream);
+                                   int ws_x, int shift_y, int shift_x, float scale, int q_prescaled, int64_t tok_stride,
+                                   int64_t head_stride, int64_t part_stride, hipStream_t stream);
 hipError_t attention_launch(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
                             int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
-                            int64_t tok_stride, int64_t head_stride, int64_t part_stride, hipStream_t stream);
+                            int q_prescaled, int64_t tok_stride, int64_t head_stride, int64_t part_stride,
+                            hipStream_t stream);
 
 bool norm_supported(int d);
 hipError_t norm_modulate_launch(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,

@@ -41,6 +41,7 @@ struct AttnParams {
   int sy, sx;
   int use_mask;
   float scale;
+  int q_prescaled;  // q already holds q * scale * log2(e) (the producing GEMM scaled it in fp32 before its only rounding)
 };
 
 template <int WS_Y, int WS_X, int HD, bool HAS_BIAS>
@@ -212,9 +213,9 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     }
     // tail components R4[s][e] with s+e >= TBL are never read by a valid key group
   }
-  // ---- q * scale * log2(e), rounded to bf16 once more: the accumulators of K Q^T are then the logits in the exp2
-  // domain and P = exp2(acc) needs no multiply
-  {
+  // ---- q * scale * log2(e), rounded to bf16 once more (unless the producer of q has applied the factor already): the
+  // accumulators of K Q^T are then the logits in the exp2 domain and P = exp2(acc) needs no multiply
+  if (!p.q_prescaled) {
     const float c = p.scale * LOG2E;
 #pragma unroll
     for (int ps = 0; ps < 2; ++ps)
@@ -566,7 +567,7 @@ window_attention_dma_kernel(AttnParams p) {
     }
   }
   // ---- q * scale * log2(e): the accumulators of K Q^T are then the logits in the exp2 domain
-  {
+  if (!p.q_prescaled) {
     const float c = p.scale * LOG2E;
 #pragma unroll
     for (int ps = 0; ps < 2; ++ps)
@@ -983,6 +984,7 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
     }
     // this wave's loads of unit u (and its bias writes) have landed; only the 4 output stores of the unit before may
     // still be outstanding (vector memory operations complete in order)
+    static_assert(DB * 2 == 4, "the vmcnt(4) below counts the DB * 2 output stores a wave issues per unit");
     if (u == u_begin) __builtin_amdgcn_s_waitcnt(0x0070);
     else __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
@@ -1003,11 +1005,15 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
     const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
     bf16x8 qf[KS];
 #pragma unroll
-    for (int s2 = 0; s2 < KS; ++s2) {
-      u32x4 w = __builtin_bit_cast(u32x4, q_cur[s2]);
+    for (int s2 = 0; s2 < KS; ++s2) qf[s2] = q_cur[s2];
+    if (!p.q_prescaled) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(bf16_lo(w[e]) * cq, bf16_hi(w[e]) * cq);
-      qf[s2] = __builtin_bit_cast(bf16x8, w);
+      for (int s2 = 0; s2 < KS; ++s2) {
+        u32x4 w = __builtin_bit_cast(u32x4, q_cur[s2]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(bf16_lo(w[e]) * cq, bf16_hi(w[e]) * cq);
+        qf[s2] = __builtin_bit_cast(bf16x8, w);
+      }
     }
 
     auto init_acc = [&](int kb, f32x16& a) {
@@ -1262,8 +1268,10 @@ static hipError_t launch_attn(const AttnParams& p, hipStream_t stream) {
 
 hipError_t attention_launch(const void* qkv, void* out, const void* bias_table, int B, int H, int W, int heads,
                             int head_dim, int ws_y, int ws_x, int shift_y, int shift_x, int use_mask, float scale,
-                            int64_t tok_stride, int64_t head_stride, int64_t part_stride, hipStream_t stream) {
+                            int q_prescaled, int64_t tok_stride, int64_t head_stride, int64_t part_stride,
+                            hipStream_t stream) {
   AttnParams p;
+  p.q_prescaled = q_prescaled;
   p.tok_stride = tok_stride; p.head_stride = head_stride; p.part_stride = part_stride;
   p.qkv = reinterpret_cast<const uint16_t*>(qkv);
   p.out = reinterpret_cast<uint16_t*>(out);

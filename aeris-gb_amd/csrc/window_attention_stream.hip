@@ -35,6 +35,7 @@ struct StreamParams {
   int sy, sx;
   int n_units, qblks;
   float scale;
+  int q_prescaled;  // q already holds q * scale * log2(e)
   uint32_t span_bytes;  // DMA form: bytes of one image's k (or v) plane that a token offset can reach, < 2^32
 };
 
@@ -146,8 +147,9 @@ window_attention_stream_kernel(StreamParams p) {
   }
   {
     // q is multiplied by scale * log2(e) once, here (the reference scales q in bf16 too, model.py:290): the
-    // accumulators of K Q^T are then the logits in the exp2 domain and no score needs a multiply
-    const float c = p.scale * LOG2E;
+    // accumulators of K Q^T are then the logits in the exp2 domain and no score needs a multiply.  q_prescaled: the
+    // producer of q has applied the factor in fp32 before its only rounding, and this is a multiplication by one
+    const float c = p.q_prescaled ? 1.0f : p.scale * LOG2E;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const u32x4 w = __builtin_bit_cast(u32x4, qf[s]);
@@ -483,9 +485,10 @@ hipError_t attention_stream_configure_all() {
 }
 
 hipError_t attention_stream_launch(const void* qkv, void* out, int B, int H, int W, int heads, int head_dim, int ws_y,
-                                   int ws_x, int shift_y, int shift_x, float scale, int64_t tok_stride, int64_t head_stride,
-                                   int64_t part_stride, hipStream_t stream) {
+                                   int ws_x, int shift_y, int shift_x, float scale, int q_prescaled, int64_t tok_stride,
+                                   int64_t head_stride, int64_t part_stride, hipStream_t stream) {
   StreamParams p;
+  p.q_prescaled = q_prescaled;
   p.tok_stride = tok_stride; p.head_stride = head_stride; p.part_stride = part_stride;
   p.qkv = reinterpret_cast<const uint16_t*>(qkv);
   p.out = reinterpret_cast<uint16_t*>(out);

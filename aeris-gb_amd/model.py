@@ -193,13 +193,16 @@ class Attention(nn.Module):
         """y bf16 [b, n, d] -> attention output before ``wo`` (bf16 [b*n, inner])."""
         b, n, _ = y.shape
         # q, k, v leave the GEMM as one [b*n, head_dim] plane per part and head (the "(c h d) -> c h d" split of
-        # model.py:300 done by the store addresses): a window's rows are then contiguous runs for the attention kernel
+        # model.py:300 done by the store addresses): a window's rows are then contiguous runs for the attention kernel.
+        # The q planes leave the GEMM multiplied by scale * log2(e) in fp32 (model.py:290's `q * self.scale`, in the
+        # exp2 domain of the kernel's softmax) so that q is rounded to bf16 once, not twice.
         qkv = ops.gemm_heads(y, self.to_qkv.weight, self.to_qkv.bias, self.head_dim,
-                             out=ops.workspace("qkv", (3 * self.heads, b * n, self.head_dim), torch.bfloat16, y.device))
+                             out=ops.workspace("qkv", (3 * self.heads, b * n, self.head_dim), torch.bfloat16, y.device),
+                             q_scale=self.scale * ops.LOG2E, q_planes=self.heads)
         return ops.window_attention(qkv, b, self.image_shape, self.heads, self.head_dim,
                                     self.window_size, shift, self.relative_position_bias_table,
                                     self.shift_mask and (shift[0] > 0 or shift[1] > 0), self.scale, out=out,
-                                    head_planes=True)
+                                    head_planes=True, q_prescaled=True)
 
     def forward(self, x, shift=(0, 0)):
         b, n, d = x.shape

@@ -144,11 +144,12 @@ def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], he
                      window_size: Tuple[int, int], shift: Tuple[int, int] = (0, 0),
                      bias_table: Optional[torch.Tensor] = None, use_mask: bool = False,
                      scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
-                     head_planes: bool = False) -> torch.Tensor:
+                     head_planes: bool = False, q_prescaled: bool = False) -> torch.Tensor:
     """qkv bf16 [B*H*W, 3*heads*head_dim] (natural token order) -> bf16 [B*H*W, heads*head_dim].
 
     ``head_planes``: qkv is [3*heads, B*H*W, head_dim] instead (plane c*heads + h = part c of head h), the layout
-    ``gemm_heads`` writes."""
+    ``gemm_heads`` writes.  ``q_prescaled`` (head planes only): the q planes already hold q * scale * log2(e), as
+    ``gemm_heads(..., q_scale=scale * LOG2E, q_planes=heads)`` writes them."""
     H, W = image_shape
     inner = heads * head_dim
     _dev(qkv, "qkv", torch.bfloat16)
@@ -156,6 +157,8 @@ def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], he
         raise RuntimeError(f"qkv has {qkv.numel()} elements, expected {B}*{H}*{W}*3*{inner}")
     if head_planes and tuple(qkv.shape) != (3 * heads, B * H * W, head_dim):
         raise RuntimeError(f"qkv planes must be [{3 * heads}, {B * H * W}, {head_dim}], got {tuple(qkv.shape)}")
+    if q_prescaled and not head_planes:
+        raise RuntimeError("q_prescaled needs head_planes=True (the row-matrix entry point scales q itself)")
     if bias_table is not None:
         _dev(bias_table, "bias_table", torch.bfloat16)
         n = (2 * window_size[0] - 1) * (2 * window_size[1] - 1)
@@ -172,7 +175,8 @@ def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], he
         if head_planes:
             L.call("aeris_window_attention_heads_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads,
                    head_dim, window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
-                   float(head_dim ** -0.5 if scale is None else scale), B * H * W * head_dim, _stream())
+                   float(head_dim ** -0.5 if scale is None else scale), int(bool(q_prescaled)), B * H * W * head_dim,
+                   _stream())
         else:
             L.call("aeris_window_attention_fwd", qkv.data_ptr(), out.data_ptr(), _ptr(bias_table), B, H, W, heads, head_dim,
                    window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
@@ -308,9 +312,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     return out
 
 
+LOG2E = 1.4426950408889634
+
+
 def gemm_heads(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], head_dim: int,
-               out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """a[M, K] @ w[N, K]^T + bias as N / head_dim planes: bf16 [N / head_dim, M, head_dim] (see aeris_gemm_heads_fwd)."""
+               out: Optional[torch.Tensor] = None, q_scale: float = 1.0, q_planes: int = 0) -> torch.Tensor:
+    """a[M, K] @ w[N, K]^T + bias as N / head_dim planes: bf16 [N / head_dim, M, head_dim] (see aeris_gemm_heads_fwd).
+    The first ``q_planes`` planes are multiplied by ``q_scale`` in fp32 before the rounding to bf16."""
     _dev(a, "a", torch.bfloat16)
     _dev(w, "w", torch.bfloat16)
     K = a.shape[-1]
@@ -333,7 +341,7 @@ def gemm_heads(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], h
     big = gemm_uses_big_tiles(M, N, None)
     with _timed("gemm_256x256_none_bf16_plain" if big else "gemm_128x128", 2.0 * M * N * K, "flop"):
         L.call("aeris_gemm_heads_fwd", a.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(bias), M, N, K, head_dim,
-               M * head_dim, _stream())
+               M * head_dim, float(q_scale), int(q_planes), _stream())
     return out
 
 

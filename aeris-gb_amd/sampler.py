@@ -149,9 +149,19 @@ class TrigFlowSampler:
         self._out = self._captured
         return self
 
-    def _capture(self, fn, warmup, generator=None):
+    @staticmethod
+    def _side_stream():
+        """A fresh stream for warm-up work, entered only once the current stream has drained.  The block intermediates
+        are shared per device and change hands between streams only when their last user has nothing pending
+        (ops.workspace); an event wait alone would order the two streams correctly but leave that check to timing."""
+        cur = torch.cuda.current_stream()
+        cur.synchronize()
         side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
+        side.wait_stream(cur)
+        return side
+
+    def _capture(self, fn, warmup, generator=None):
+        side = self._side_stream()
         with torch.cuda.stream(side):
             for _ in range(warmup):
                 fn()
@@ -194,7 +204,7 @@ class TrigFlowSampler:
         """Set up an autoregressive forecast (arguments: see ``rollout``) and, with ``use_graph``, capture
         ``graph_steps`` consecutive forecast steps as one HIP graph (1: the graph is one forecast step and is replayed
         per step; n_forecast: the whole rollout is one graph and one replay), after ``graph_warmup`` eager steps whose
-        effect on the state is undone.  The forecast-step counter, the forcings and the state store are indexed on the
+        effect on the state, the step counter and the generator is undone.  The forecast-step counter, the forcings and the state store are indexed on the
         device, so the same recorded step serves every position of the rollout.  ``run()`` of the returned object
         advances it; ``reset()`` puts it back to ``state0`` and step 0."""
         if not 0 <= graph_warmup <= n_forecast:
@@ -209,13 +219,19 @@ class TrigFlowSampler:
         if use_graph:
             # the default generator is registered with every graph; any other one has to be registered by hand
             own = gen if gen is not None and gen is not torch.cuda.default_generators[state0.device.index or 0] else None
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                for _ in range(graph_warmup):
-                    ro.step()
-            torch.cuda.current_stream().wait_stream(side)
-            ro.reset()
+            if graph_warmup:
+                # the warm-up steps draw latents like any other step: the generator is put back afterwards, so that a
+                # seeded rollout gives the same forecast with and without warm-up, eager or replayed
+                rng = gen.get_state() if gen is not None else None
+                side = self._side_stream()
+                with torch.cuda.stream(side):
+                    for _ in range(graph_warmup):
+                        ro.step()
+                torch.cuda.current_stream().wait_stream(side)
+                side.synchronize()
+                if rng is not None:
+                    gen.set_state(rng)
+                ro.reset()
 
             def steps():
                 for _ in range(graph_steps):

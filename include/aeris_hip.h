@@ -94,10 +94,13 @@ int aeris_window_attention_fwd(const void* qkv, void* out, const void* bias_tabl
  * the planes plane_stride elements apart (what aeris_gemm_heads_fwd writes).  A window's keys are then runs of
  * ws_x * head_dim contiguous elements instead of head_dim-element pieces a whole qkv row apart: about 13 % faster at
  * 16x16 windows on the 720x1440 grid.  Same arithmetic, bit-identical output.  The layout is internal to this library: it
- * replaces the intermediate of model.py:299-302, which the reference never exposes. */
+ * replaces the intermediate of model.py:299-302, which the reference never exposes.
+ * q_prescaled != 0: the q planes already hold q * scale * log2(e), as aeris_gemm_heads_fwd writes them when it is given
+ * q_scale = scale * log2(e): the factor of model.py:290 is then applied once, in fp32, before q's only rounding to bf16,
+ * and the kernel uses q as it is (`scale` is ignored apart from its validity check). */
 int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const void* bias_table, int B, int H, int W,
                                      int heads, int head_dim, int ws_y, int ws_x, int shift_y, int shift_x,
-                                     int use_mask, float scale, int64_t plane_stride, void* stream);
+                                     int use_mask, float scale, int q_prescaled, int64_t plane_stride, void* stream);
 
 /* Row norm fused with noise-level modulation.
  *   x  [B*rows_per_batch, d] (x_dtype bf16|f32)  ->  y [B*rows_per_batch, d] (y_dtype bf16|f32)
@@ -161,9 +164,12 @@ int aeris_gemm_fwd(const void* A, const void* W, void* C, const void* bias, cons
 /* C = A[M,K] * W[N,K]^T + bias written as N / head_dim planes of bf16 [M, head_dim], plane j = columns
  * [j*head_dim, (j+1)*head_dim), the planes plane_stride elements apart (>= M * head_dim, multiple of 8).
  * The to_qkv Linear (model.py:284,299) writing the layout aeris_window_attention_heads_fwd reads; the rearrange at
- * model.py:300 ("(c h d) -> c h d") is this split.  Requires K % 64 == 0, head_dim % 8 == 0, N % head_dim == 0. */
+ * model.py:300 ("(c h d) -> c h d") is this split.  Requires K % 64 == 0, head_dim % 8 == 0, N % head_dim == 0.
+ * The first q_planes planes (the query part; 0 = none) are multiplied by q_scale in fp32 after the bias and before the
+ * rounding to bf16: with q_scale = head_dim^-0.5 * log2(e) this is the `q * self.scale` of model.py:290 in the exp2
+ * domain, and aeris_window_attention_heads_fwd takes such planes with q_prescaled = 1. */
 int aeris_gemm_heads_fwd(const void* A, const void* W, void* C, const void* bias, int64_t M, int N, int K,
-                         int head_dim, int64_t plane_stride, void* stream);
+                         int head_dim, int64_t plane_stride, float q_scale, int q_planes, void* stream);
 
 /* y[b, n] = act(sum_k x[b,k] * W[n,k] + bias[n]);  x f32 [B,K], W bf16|f32 [N,K], bias same type or NULL,
  * y f32 [B,N].  The two Linear layers of ModulationLinear (model.py:311-325) with SiLU in between. */

@@ -21,8 +21,11 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def depth_curve(pkg, cuda, cfg, preset, res_dt, seed, grid_tokens, dt_value=0.9, use_ape=False):
-    sd = oracle.init_model_weights(cfg, seed)  # the benchmark's init: trunc-normal(0.02) matrices, zero biases, unit gains
+def depth_curve(pkg, cuda, cfg, preset, res_dt, seed, grid_tokens, dt_value=0.9, use_ape=False, nontrivial=False):
+    # nontrivial False: the benchmark's init, trunc-normal(0.02) matrices, zero biases, unit norm gains (every branch
+    # adds little to the stream).  True: unit-gain matrices, perturbed biases and gains, gates near 1: every branch
+    # adds a term as large as the stream itself, the way a trained checkpoint's blocks do
+    sd = oracle.init_model_weights(cfg, seed, nontrivial=nontrivial)
     model = make_model(pkg, cfg, sd, cuda, res_dt, preset)
     g = torch.Generator().manual_seed(seed + 1)
     x, dt = torch.randn(1, grid_tokens, cfg.in_channels, generator=g), torch.tensor([dt_value])
@@ -57,16 +60,22 @@ def report(tag, curve, final, extra):
         pass
 
 
-@pytest.mark.parametrize("res_dt", [torch.bfloat16, torch.float32], ids=["bf16_residual", "f32_residual"])
-def test_config3_depth_24_blocks(pkg, cuda, res_dt):
+@pytest.mark.parametrize("res_dt,seed,nontrivial", [
+    (torch.bfloat16, 3, False), (torch.float32, 3, False), (torch.float32, 3, True), (torch.float32, 11, False),
+    (torch.float32, 11, True)], ids=["bf16_residual", "f32_residual", "f32_residual_unit_gain", "f32_residual_seed11",
+                                     "f32_residual_unit_gain_seed11"])
+def test_config3_depth_24_blocks(pkg, cuda, res_dt, seed, nontrivial):
     """configs[3]'s denoiser (138 -> dim 1536 -> 24 blocks of 24 x 64 heads, 16x16 windows alternately un-shifted and
-    shifted by 8 with mask and rel-pos bias, LayerNorm + scale/shift modulation, GELU MLP 6144 -> 69) on a 64x128 grid."""
+    shifted by 8 with mask and rel-pos bias, LayerNorm + scale/shift modulation, GELU MLP 6144 -> 69) on a 64x128 grid;
+    with the benchmark's init and with unit-gain weights (every branch output as large as the stream), two seeds."""
     H, W = 64, 128
     cfg = OracleConfig.spec(n_layers=26, in_channels=138, out_channels=69, dim=1536, heads=24, head_dim=64, mlp_dim=6144,
                             window_size=(16, 16), image_shape=(H, W), mod_ways=2)
-    curve, final = depth_curve(pkg, cuda, cfg, "spec", res_dt, 3, H * W)
-    tag = "config3_" + ("bf16" if res_dt == torch.bfloat16 else "f32") + "_residual"
-    report(tag, curve, final, {"grid": [H, W], "preset": "spec, mod_ways 2", "blocks": 24, "dim": 1536})
+    curve, final = depth_curve(pkg, cuda, cfg, "spec", res_dt, seed, H * W, nontrivial=nontrivial)
+    tag = ("config3_" + ("bf16" if res_dt == torch.bfloat16 else "f32") + "_residual" + ("_unit_gain" if nontrivial else "")
+           + (f"_seed{seed}" if seed != 3 else ""))
+    report(tag, curve, final, {"grid": [H, W], "preset": "spec, mod_ways 2", "blocks": 24, "dim": 1536, "seed": seed,
+                               "unit_gain_weights": nontrivial})
     if res_dt == torch.float32:  # the default residual stream of LocalAERIS: inside the tolerance at every depth
         assert final["rel_l2"] <= 1e-2, final
         assert max(c["rel_l2"] for c in curve) <= 1e-2, curve
@@ -78,13 +87,17 @@ def test_config3_depth_24_blocks(pkg, cuda, res_dt):
         assert final["rel_l2"] <= 2e-2, final
 
 
-def test_reference_block_depth_24_blocks(pkg, cuda):
+@pytest.mark.parametrize("seed,nontrivial", [(5, False), (5, True), (12, True)], ids=["init", "unit_gain", "unit_gain_seed12"])
+def test_reference_block_depth_24_blocks(pkg, cuda, seed, nontrivial):
     """The reference's own model shape (model.py:358-403, train.yaml: dim 1536, 12 heads x 128, SwiGLU 6144, 60x60 windows,
-    8 layers x 3 sublayers = 24 blocks, RMSNorm, 6-way modulation before the norm, APE on the inputs) on a 120x120 grid."""
+    8 layers x 3 sublayers = 24 blocks, RMSNorm, 6-way modulation before the norm, APE on the inputs) on a 120x120 grid;
+    with the benchmark's init (gates near 0) and with unit-gain weights and gates near 1, two seeds."""
     H, W = 120, 120
     cfg = OracleConfig.ref(n_layers=10, sublayers=3, in_channels=144, out_channels=70, dim=1536, heads=12, head_dim=128,
                            mlp_dim=6144, window_size=(60, 60), image_shape=(H, W))
-    curve, final = depth_curve(pkg, cuda, cfg, "ref", torch.float32, 5, H * W, use_ape=True)
-    report("refwin_f32_residual", curve, final, {"grid": [H, W], "preset": "ref", "blocks": 24, "dim": 1536})
+    curve, final = depth_curve(pkg, cuda, cfg, "ref", torch.float32, seed, H * W, use_ape=True, nontrivial=nontrivial)
+    tag = "refwin_f32_residual" + ("_unit_gain" if nontrivial else "") + (f"_seed{seed}" if seed != 5 else "")
+    report(tag, curve, final, {"grid": [H, W], "preset": "ref", "blocks": 24, "dim": 1536, "seed": seed,
+                               "unit_gain_weights": nontrivial})
     assert final["rel_l2"] <= 1e-2, final
     assert max(c["rel_l2"] for c in curve) <= 1e-2, curve

@@ -179,31 +179,47 @@ PLANE_CASES = [
 ]
 
 
+LOG2E = 1.4426950408889634
+
+
+@pytest.mark.parametrize("prescaled", [True, False], ids=["qscaled", "qraw"])
 @pytest.mark.parametrize("case", PLANE_CASES, ids=lambda c: f"B{c[0]}_{c[1]}x{c[2]}_h{c[3]}x{c[4]}_ws{c[5]}_s{c[6]}_b{int(c[7])}m{int(c[8])}_x{c[9]:g}")
-def test_window_attention_planes_parity(pkg, cuda, case):
+def test_window_attention_planes_parity(pkg, cuda, case, prescaled):
+    """``prescaled``: the q planes hold bf16(q * scale * log2 e), the form the to_qkv GEMM of the model writes (the
+    factor applied in fp32 before q's only rounding); the oracle is given exactly those queries (divided by the factor
+    again, in fp32), so what is compared is the kernel's own arithmetic: P and O rounded to bf16 once each, at any
+    logit magnitude.  Not prescaled: the kernel multiplies the bf16 q by the factor and rounds again (as the
+    reference's bf16 `q * self.scale` does, model.py:290), which moves a logit by 2^-9 of its magnitude: nothing at
+    ordinary magnitudes, a few percent of P once logits reach the hundreds."""
     B, H, W, heads, hd, ws, sh, has_bias, use_mask, mag = case
     g = torch.Generator().manual_seed(H * W + heads + int(mag))
     inner, S = heads * hd, B * H * W
     qkv = torch.randn(B, H * W, 3 * inner, generator=g)
     qkv[..., :2 * inner] *= mag  # logits of magnitude mag^2 * sqrt(hd) * scale: up to several hundred, and as far below zero
-    qkv = bf(qkv)
+    c = hd ** -0.5 * LOG2E
+    if prescaled:
+        q_dev = bf(qkv[..., :inner] * c)
+        kv = bf(qkv[..., inner:])
+        dev_in = torch.cat([q_dev, kv], dim=-1)
+        ref_in = torch.cat([q_dev.float() / c, kv.float()], dim=-1)
+    else:
+        dev_in = bf(qkv)
+        ref_in = dev_in.float()
     table = bf(0.7 * torch.randn((2 * ws - 1) ** 2, heads, generator=g)) if has_bias else None
     cfg = OracleConfig(dim=inner, heads=heads, head_dim=hd, mlp_dim=inner, window_size=(ws, ws), image_shape=(H, W),
                        rel_pos_bias=has_bias, shift_mask=use_mask)
-    ref = attention_core(cfg, qkv.float(), (sh, sh), None if table is None else table.float())
-    planes = qkv.view(S, 3 * heads, hd).permute(1, 0, 2).contiguous().to(cuda)  # plane c * heads + h = part c of head h
+    ref = attention_core(cfg, ref_in, (sh, sh), None if table is None else table.float())
+    planes = dev_in.view(S, 3 * heads, hd).permute(1, 0, 2).contiguous().to(cuda)  # plane c * heads + h = part c of head h
     out = pkg.ops.window_attention(planes, B, (H, W), heads, hd, (ws, ws), (sh, sh), None if table is None else table.to(cuda),
-                                   use_mask, head_planes=True)
+                                   use_mask, head_planes=True, q_prescaled=prescaled)
     out2 = pkg.ops.window_attention(planes, B, (H, W), heads, hd, (ws, ws), (sh, sh), None if table is None else table.to(cuda),
-                                    use_mask, head_planes=True)
+                                    use_mask, head_planes=True, q_prescaled=prescaled)
     torch.cuda.synchronize()
     assert torch.equal(out, out2)
     assert bool(torch.isfinite(out.float()).all())
     err = rel_l2(out.view(B, H * W, inner), ref)
-    # P and O are rounded to bf16 once each, and q once more after it is multiplied by the scale (as in the reference,
-    # whose `q * self.scale` is a bf16 product, model.py:290): that rounding moves a logit by 2^-9 of its magnitude,
-    # which is nothing at ordinary magnitudes and a few percent of P once logits reach the hundreds
-    assert err <= (6e-3 if mag == 1.0 else 3e-2), err
+    print(f"planes attention, |q|,|k| x{mag}, prescaled {prescaled}: rel-L2 {err:.3e}")
+    assert err <= (6e-3 if (mag == 1.0 or prescaled) else 3e-2), err
     if mag == 1.0:
         assert (out.float().cpu().view(B, H * W, inner) - ref).abs().max() < 0.06
 
@@ -266,6 +282,21 @@ def test_window_attention_streaming_large_logits(pkg, cuda, case):
     err = rel_l2(out.view(B, H * W, inner), ref)
     print(f"streaming attention, |q|,|k| x{mag}: rel-L2 {err:.3e}")
     assert err <= 3e-2, err
+    # the same queries handed over as head planes that already hold bf16(q * scale * log2 e) (what the model's to_qkv
+    # GEMM writes): q is rounded once, and the oracle on exactly those queries is met at the ordinary tolerance
+    S = B * H * W
+    c = hd ** -0.5 * LOG2E
+    raw = torch.randn(B, H * W, 3 * inner, generator=torch.Generator().manual_seed(int(mag * 10) + hd))
+    raw[..., :2 * inner] *= mag
+    q_dev, kv = bf(raw[..., :inner] * c), bf(raw[..., inner:])
+    ref = attention_core(cfg, torch.cat([q_dev.float() / c, kv.float()], dim=-1), (ws // 2, ws // 2), None)
+    planes = torch.cat([q_dev, kv], dim=-1).view(S, 3 * heads, hd).permute(1, 0, 2).contiguous().to(cuda)
+    out = pkg.ops.window_attention(planes, B, (H, W), heads, hd, (ws, ws), (ws // 2, ws // 2), None, False, head_planes=True,
+                                   q_prescaled=True)
+    torch.cuda.synchronize()
+    err = rel_l2(out.view(B, H * W, inner), ref)
+    print(f"streaming attention, |q|,|k| x{mag}, q prescaled: rel-L2 {err:.3e}")
+    assert bool(torch.isfinite(out).all()) and err <= 6e-3, err
 
 
 def test_window_attention_streaming_wide_rows_match_compact(pkg, cuda):
@@ -323,6 +354,82 @@ def test_head_plane_layout_is_bit_identical(pkg, cuda, case):
     o2 = pkg.ops.window_attention(planes, B, (H, W), heads, hd, (wsy, wsx), (sh, sh), table, use_mask, head_planes=True)
     torch.cuda.synchronize()
     assert torch.isfinite(o1).all() and torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize("shape", [(160 * 160, 24, 64), (32 * 64, 4, 32), (24 * 24, 3, 64)], ids=["persistent", "hd32", "small"])
+def test_gemm_heads_scales_the_query_planes_in_fp32(pkg, cuda, shape):
+    """q_scale / q_planes of gemm_heads: the key and value planes are untouched bit for bit; a query plane is the fp32
+    result times the factor, rounded once - within one bf16 ulp of (rounded result) * factor, and for a factor that is a
+    power of two exactly equal to it."""
+    S, heads, hd = shape
+    g = torch.Generator().manual_seed(S + heads)
+    inner, K = heads * hd, 128
+    x = bf(torch.randn(S, K, generator=g)).to(cuda)
+    w = bf(torch.randn(3 * inner, K, generator=g) / math.sqrt(K)).to(cuda)
+    bias = bf(0.3 * torch.randn(3 * inner, generator=g)).to(cuda)
+    plain = pkg.ops.gemm_heads(x, w, bias, hd)
+    for c in (hd ** -0.5 * LOG2E, 0.25):
+        scaled = pkg.ops.gemm_heads(x, w, bias, hd, q_scale=c, q_planes=heads)
+        torch.cuda.synchronize()
+        assert torch.equal(scaled[heads:], plain[heads:])
+        want = plain[:heads].float() * c
+        if c == 0.25:
+            assert torch.equal(scaled[:heads].float(), want)
+        else:
+            assert bool(((scaled[:heads].float() - want).abs() <= want.abs() * 2.0 ** -7 + 1e-30).all())
+            ref = (x.float() @ w[:inner].float().T + bias[:inner].float()) * c  # fp32 throughout, one rounding at the end
+            got = scaled[:heads].permute(1, 0, 2).reshape(S, inner).float()
+            assert rel_l2(got.cpu(), ref.cpu()) <= 2.5e-3  # one bf16 rounding: 2^-9 / sqrt(3) = 1.1e-3 on average
+
+
+NONFINITE_CASES = [
+    # B, H, W, heads, hd, ws, shift, bias + mask, head planes -- one case per kernel form
+    ("persistent", 1, 160, 160, 24, 64, 16, 8, True, True),
+    ("one_unit_dma", 3, 32, 48, 2, 64, 16, 8, True, True),
+    ("register_staged_rows", 1, 48, 64, 3, 64, 16, 8, True, False),
+    ("register_staged_hd32", 1, 32, 64, 4, 32, 8, 4, True, True),
+    ("streaming_rows", 2, 40, 60, 3, 64, 20, 10, False, False),
+    ("streaming_planes_hd128", 1, 120, 120, 2, 128, 60, 30, False, True),
+]
+
+
+@pytest.mark.parametrize("case", NONFINITE_CASES, ids=lambda c: c[0])
+def test_window_attention_non_finite_inputs_stay_in_their_window(pkg, cuda, case):
+    """NaN-in -> NaN-out, and nowhere else.  One token's q, k, v (all heads) are NaN and another token's, in a different
+    window, +Inf.  The kernels' fast path (no row maximum) sees row sums out of range and repeats the window in the
+    two-pass / online form; the call returns, every output of the NaN window is NaN (its key poisons every query's
+    softmax), every output of the Inf window is non-finite (Inf - Inf in the logits), and every other window is bit for
+    bit what it is on clean inputs."""
+    _, B, H, W, heads, hd, ws, sh, bias_mask, planes = case
+    g = torch.Generator().manual_seed(H + W + hd)
+    inner, S = heads * hd, B * H * W
+    qkv = bf(torch.randn(S, 3 * inner, generator=g))
+    table = bf(0.7 * torch.randn((2 * ws - 1) ** 2, heads, generator=g)).to(cuda) if bias_mask else None
+    wmap = torch.from_numpy(pkg.ops.window_index_map(B, H, W, ws, ws, sh, sh))  # [windows, L] token rows
+    n_win = wmap.shape[0]
+    w_nan, w_inf = n_win - 1, n_win // 2  # the last window lies on the wrapped, masked border of a shifted grid
+    bad = qkv.clone()
+    bad[wmap[w_nan, 5]] = float("nan")
+    bad[wmap[w_inf, wmap.shape[1] - 3]] = float("inf")
+
+    def run(t):
+        if planes:
+            t = t.view(S, 3 * heads, hd).permute(1, 0, 2).contiguous()
+        else:
+            t = t.view(S, 3 * inner)
+        return pkg.ops.window_attention(t.to(cuda), B, (H, W), heads, hd, (ws, ws), (sh, sh), table, bias_mask,
+                                        head_planes=planes)
+
+    clean, got = run(qkv), run(bad)
+    torch.cuda.synchronize()  # returns: no wave spins on a value that never becomes finite
+    assert bool(torch.isfinite(clean.float()).all())
+    rows_nan, rows_inf = wmap[w_nan].to(cuda), wmap[w_inf].to(cuda)
+    assert bool(torch.isnan(got[rows_nan].float()).all())
+    assert not bool(torch.isfinite(got[rows_inf].float()).any())
+    keep = torch.ones(S, dtype=torch.bool, device=cuda)
+    keep[rows_nan] = False
+    keep[rows_inf] = False
+    assert torch.equal(got[keep], clean[keep])
 
 
 def test_window_attention_streaming_rejects_bias_and_mask(pkg, cuda):

@@ -97,6 +97,25 @@ def test_input_stage_kernel_against_float64(pkg, cuda, case):
     assert e <= (1e-5 if out_dtype == torch.float32 else 3e-3), (e, ma)
 
 
+def test_input_stage_without_encoding_keeps_a_non_finite_input_in_its_own_token(pkg, cuda):
+    """No positional encoding: an Inf (or NaN) in the first element of the input makes token 0 non-finite, as in the
+    reference's Linear, and leaves every other token exactly what it is with a finite value there."""
+    ops = pkg.ops
+    M, C0, C1, d = 600, 20, 11, 256
+    g = torch.Generator().manual_seed(3)
+    x0, x1 = torch.randn(M, C0, generator=g), torch.randn(M, C1, generator=g)
+    w, b = torch.randn(d, C0 + C1, generator=g) * 0.1, torch.randn(d, generator=g)
+    packed = ops.input_stage_pack_weight(w.to(cuda), b.to(cuda))
+    clean = ops.input_stage(x0.to(cuda), 2.0, x1.to(cuda), None, packed, d).clone()
+    for bad in (float("inf"), float("nan")):
+        x0b = x0.clone()
+        x0b[0, 0] = bad
+        got = ops.input_stage(x0b.to(cuda), 2.0, x1.to(cuda), None, packed, d)
+        torch.cuda.synchronize()
+        assert not bool(torch.isfinite(got[0]).all())
+        assert torch.equal(got[1:], clean[1:])
+
+
 def test_input_stage_falls_back_for_wide_inputs(pkg, cuda):
     """More than 159 input channels: the operand-matrix + GEMM form, same accuracy."""
     ops = pkg.ops

@@ -103,17 +103,21 @@ def test_argument_validation_needs_no_gpu(pkg):
     assert h(p16, p16, p16, None, None, None, 8, 8, 64, 8, 9, 0, 0, 0, 0, None) == L.EINVAL  # act
     # head-plane variants: same checks, plus the plane geometry
     fh = lib.aeris_window_attention_heads_fwd
-    assert fh(None, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 256 * 64, None) == L.EINVAL
-    assert fh(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 256 * 64 - 8, None) == L.EINVAL  # planes overlap
+    assert fh(None, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 0, 256 * 64, None) == L.EINVAL
+    assert fh(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 1, 256 * 64 - 8, None) == L.EINVAL  # planes overlap
     assert "plane_stride" in L.last_error()
-    assert fh(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 256 * 64 + 4, None) == L.EINVAL  # not 16-byte planes
-    assert fh(p16, p16, None, 1, 16, 16, 2, 96, 16, 16, 0, 0, 0, 0.1, 256 * 96, None) == L.EUNSUPPORTED  # head_dim 96
+    assert fh(p16, p16, None, 1, 16, 16, 2, 64, 16, 16, 0, 0, 0, 0.125, 0, 256 * 64 + 4, None) == L.EINVAL  # not 16-byte planes
+    assert fh(p16, p16, None, 1, 16, 16, 2, 96, 16, 16, 0, 0, 0, 0.1, 0, 256 * 96, None) == L.EUNSUPPORTED  # head_dim 96
     hh = lib.aeris_gemm_heads_fwd
-    assert hh(p16, p16, p16, None, 8, 128, 100, 64, 8 * 64, None) == L.EUNSUPPORTED  # K % 64
-    assert hh(p16, p16, p16, None, 8, 100, 64, 64, 8 * 64, None) == L.EINVAL  # N % head_dim
-    assert hh(p16, p16, p16, None, 8, 128, 64, 60, 8 * 60, None) == L.EINVAL  # head_dim % 8
-    assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64 - 8, None) == L.EINVAL  # planes overlap
-    assert hh(p16, None, p16, None, 8, 128, 64, 64, 8 * 64, None) == L.EINVAL  # W NULL
+    assert hh(p16, p16, p16, None, 8, 128, 100, 64, 8 * 64, 1.0, 0, None) == L.EUNSUPPORTED  # K % 64
+    assert hh(p16, p16, p16, None, 8, 100, 64, 64, 8 * 64, 1.0, 0, None) == L.EINVAL  # N % head_dim
+    assert hh(p16, p16, p16, None, 8, 128, 64, 60, 8 * 60, 1.0, 0, None) == L.EINVAL  # head_dim % 8
+    assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64 - 8, 1.0, 0, None) == L.EINVAL  # planes overlap
+    assert hh(p16, None, p16, None, 8, 128, 64, 64, 8 * 64, 1.0, 0, None) == L.EINVAL  # W NULL
+    assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64, 0.18, 3, None) == L.EINVAL  # more query planes than planes
+    assert "q_planes" in L.last_error()
+    assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64, 0.0, 1, None) == L.EINVAL  # q_scale must be positive
+    assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64, float("nan"), 1, None) == L.EINVAL
     # fused output stage
     osf, osw = lib.aeris_output_stage_fwd, lib.aeris_output_stage_workspace_bytes
     assert osw(69, 1536, 1) == 1536 * 80 * 4 + 80 * 8 and osw(69, 1536, 4) == 4 * osw(69, 1536, 1)

@@ -31,6 +31,9 @@ SIGNATURES = {
     "aeris_shift_region_ids": (_c_int, [_c_int] * 6 + [_c_vp]),
     "aeris_window_attention_fwd": (_c_int, [_c_vp, _c_vp, _c_vp] + [_c_int] * 10 + [_c_f32, _c_vp]),
     "aeris_window_attention_heads_fwd": (_c_int, [_c_vp, _c_vp, _c_vp] + [_c_int] * 10 + [_c_f32, _c_int, _c_i64, _c_vp]),
+    "aeris_qkv_attention_bias_bytes": (_c_i64, [_c_int, _c_int, _c_int]),
+    "aeris_qkv_attention_prepare_bias": (_c_int, [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_vp]),
+    "aeris_qkv_window_attention_fwd": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp] + [_c_int] * 11 + [_c_f32, _c_vp]),
     "aeris_norm_modulate_fwd": (_c_int, [_c_vp, _c_int, _c_vp, _c_int, _c_vp, _c_vp, _c_int, _c_vp, _c_vp, _c_i64, _c_i64,
                                          _c_i64, _c_int, _c_int, _c_int, _c_f32, _c_vp]),
     "aeris_output_stage_workspace_bytes": (_c_i64, [_c_int, _c_int, _c_int]),

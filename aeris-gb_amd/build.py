@@ -15,8 +15,8 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "libaeris_hip.so")
-SOURCES = ["api.hip", "gemm.hip", "gemm_persistent.hip", "window_attention.hip", "window_attention_stream.hip", "norm_modulate.hip", "small_ops.hip", "output_stage.hip", "input_stage.hip"]
-HEADERS = ["common.h", "kernels.h", "gemm_common.h", os.path.join("..", "..", "include", "aeris_hip.h")]
+SOURCES = ["api.hip", "gemm.hip", "gemm_persistent.hip", "window_attention.hip", "qkv_window_attention.hip", "window_attention_stream.hip", "norm_modulate.hip", "small_ops.hip", "output_stage.hip", "input_stage.hip"]
+HEADERS = ["common.h", "kernels.h", "gemm_common.h", "attention_sweep.h", os.path.join("..", "..", "include", "aeris_hip.h")]
 # packed fp32 VALU ops stay off: some of their forms have produced wrong results on this hardware
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]

@@ -42,6 +42,7 @@ int ensure_init(void* stream = nullptr, bool from_launch = false) {
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_configure_all();
     if (g_init_status == hipSuccess) g_init_status = aeris::attention_stream_configure_all();
     if (g_init_status == hipSuccess) g_init_status = aeris::input_stage_configure();
+    if (g_init_status == hipSuccess) g_init_status = aeris::qkv_attention_configure();
     g_init_done.store(true, std::memory_order_release);
   });
   if (g_init_status == hipSuccess && !from_launch) {
@@ -184,6 +185,49 @@ int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const vo
   return window_attention_impl("aeris_window_attention_heads_fwd", qkv_planes, out, bias_table, B, H, W, heads, head_dim, ws_y,
                                ws_x, shift_y, shift_x, use_mask, scale, q_prescaled ? 1 : 0, head_dim, plane_stride,
                                (int64_t)heads * plane_stride, stream);
+}
+
+int64_t aeris_qkv_attention_bias_bytes(int heads, int ws_y, int ws_x) {
+  if (heads <= 0 || !aeris::qkv_attention_supported(ws_y, ws_x, 64, 128, 1)) return 0;
+  return aeris::qkv_attention_bias_bytes(heads);
+}
+
+int aeris_qkv_attention_prepare_bias(const void* bias_table, int heads, int ws_y, int ws_x, void* out, void* stream) {
+  if (!bias_table || !out) return fail(AERIS_EINVAL, "aeris_qkv_attention_prepare_bias: bias_table/out is NULL");
+  if (heads <= 0) return fail(AERIS_EINVAL, "aeris_qkv_attention_prepare_bias: heads must be positive");
+  if (!aeris::qkv_attention_supported(ws_y, ws_x, 64, 128, 1))
+    return fail(AERIS_EUNSUPPORTED, "aeris_qkv_attention_prepare_bias: only 16x16 windows are built (got %dx%d)", ws_y, ws_x);
+  if (!aligned16(out)) return fail(AERIS_EINVAL, "aeris_qkv_attention_prepare_bias: out must be 16-byte aligned");
+  hipError_t e = aeris::qkv_attention_bias_launch(bias_table, reinterpret_cast<float*>(out), heads, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_qkv_attention_prepare_bias launch");
+  return AERIS_OK;
+}
+
+int aeris_qkv_window_attention_fwd(const void* y, const void* w, const void* qkv_bias, const void* bias4, void* out, int B,
+                                   int H, int W, int heads, int head_dim, int K, int ws_y, int ws_x, int shift_y, int shift_x,
+                                   int use_mask, float scale, void* stream) {
+  const char* who = "aeris_qkv_window_attention_fwd";
+  if (!y || !w || !out) return fail(AERIS_EINVAL, "%s: y/w/out is NULL", who);
+  if (!aligned16(y) || !aligned16(w) || !aligned16(out) || (bias4 && !aligned16(bias4)))
+    return fail(AERIS_EINVAL, "%s: y/w/out/bias4 must be 16-byte aligned", who);
+  if (qkv_bias && (reinterpret_cast<uintptr_t>(qkv_bias) & 7u)) return fail(AERIS_EINVAL, "%s: qkv_bias must be 8-byte aligned", who);
+  if (heads <= 0 || head_dim <= 0 || K <= 0) return fail(AERIS_EINVAL, "%s: heads, head_dim, K must be positive", who);
+  if (int rc = check_window_geometry(B, H, W, ws_y, ws_x, shift_y, shift_x)) return rc;
+  if (!(scale > 0.f)) return fail(AERIS_EINVAL, "%s: scale must be positive", who);
+  if (!aeris::qkv_attention_supported(ws_y, ws_x, head_dim, K, (int64_t)H * W))
+    return fail(AERIS_EUNSUPPORTED,
+                "%s: built for 16x16 windows, head_dim 64, K a multiple of 128 and H*W*K*2 < 2^32 (got %dx%d, head_dim %d, "
+                "K %d, H*W %lld): use aeris_gemm_heads_fwd + aeris_window_attention_heads_fwd", who, ws_y, ws_x, head_dim, K,
+                (long long)H * W);
+  if ((int64_t)3 * heads * head_dim * K * 2 >= (int64_t(1) << 31))
+    return fail(AERIS_EUNSUPPORTED, "%s: the to_qkv weight must be smaller than 2 GiB", who);
+  if ((int64_t)B * (H / ws_y) * (W / ws_x) * heads > 0x7fffffffLL || (int64_t)B * H * W > 0x7fffffffLL)
+    return fail(AERIS_EUNSUPPORTED, "%s: more than 2^31-1 (window, head) units or tokens", who);
+  if (int rc = ensure_init(stream, true)) return rc;
+  hipError_t e = aeris::qkv_attention_launch(y, w, qkv_bias, reinterpret_cast<const float*>(bias4), out, B, H, W, heads, K, shift_y,
+                                             shift_x, use_mask, scale, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "aeris_qkv_window_attention_fwd launch");
+  return AERIS_OK;
 }
 
 int aeris_norm_modulate_fwd(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,

@@ -48,6 +48,35 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// ---- ds_read_b64_tr_b16 (the LDS read that transposes 4 x 4 blocks of 16-bit elements on the way out) as inline assembly.
+// The compiler's builtin form may not be used while a buffer_load ... lds is in flight: the compiler cannot tell that
+// the read does not alias the load's destination and puts an s_waitcnt vmcnt(0) in front of it, which makes a wave
+// wait for the next unit's (or chunk's) loads in the middle of the arithmetic that they are meant to run under.
+// The assembly form is invisible to that analysis - and to the compiler's count of outstanding LDS operations: the
+// result registers must pass through lds_tr_wait() (s_waitcnt lgkmcnt(0)) before anything reads them.  ("memory"
+// keeps the compiler from moving LDS accesses of its own across the read; its own lgkmcnt waits stay correct, LDS
+// operations return in order and extra outstanding ones only make a counted wait stricter.)
+__device__ __forceinline__ uint32_t lds_byte_address(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+template <int OFFSET>
+__device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t lds_address) {
+  u32x2 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(lds_address), "n"(OFFSET) : "memory");
+  return r;
+}
+struct TrFrag { u32x2 lo, hi; };  // two transposing reads = the 8 k slots of one MFMA operand
+__device__ __forceinline__ void lds_tr_wait(TrFrag& a, TrFrag& b) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi));
+}
+__device__ __forceinline__ void lds_tr_wait(TrFrag& a, TrFrag& b, TrFrag& c, TrFrag& d) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi), "+v"(c.lo), "+v"(c.hi), "+v"(d.lo), "+v"(d.hi));
+}
+__device__ __forceinline__ bf16x8 tr_frag_value(const TrFrag& f) {
+  return __builtin_bit_cast(bf16x8, u32x4{f.lo.x, f.lo.y, f.hi.x, f.hi.y});
+}
+
 __device__ __forceinline__ float silu_f(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 __device__ __forceinline__ float erf_poly(float x) {
   // Abramowitz-Stegun 7.1.26, abs error <= 1.5e-7 (below bf16 and fp32-accumulation noise)

@@ -29,6 +29,15 @@ hipError_t attention_launch(const void* qkv, void* out, const void* bias_table, 
                             int q_prescaled, int64_t tok_stride, int64_t head_stride, int64_t part_stride,
                             hipStream_t stream);
 
+// to_qkv projection fused with window attention (qkv_window_attention.hip): 16x16 windows, head_dim 64, K % 128 == 0
+bool qkv_attention_supported(int ws_y, int ws_x, int head_dim, int K, int64_t tokens_per_image);
+int64_t qkv_attention_bias_bytes(int heads);
+hipError_t qkv_attention_configure();
+hipError_t qkv_attention_bias_launch(const void* table, float* out, int heads, hipStream_t stream);
+hipError_t qkv_attention_launch(const void* y, const void* w, const void* bias, const float* bias4, void* out, int B, int H,
+                                int W, int heads, int K, int shift_y, int shift_x, int use_mask, float scale,
+                                hipStream_t stream);
+
 bool norm_supported(int d);
 hipError_t norm_modulate_launch(const void* x, int x_dtype, void* y, int y_dtype, const void* gamma, const void* beta,
                                 int param_dtype, const float* shift, const float* scale, int64_t mod_batch_stride, int64_t B,

@@ -25,6 +25,7 @@
 // step ahead of their use); q / k / v are addressed through strides, so they may be the columns of one [tokens, 3*inner]
 // matrix or one [tokens, head_dim] plane per part and head.
 #include "common.h"
+#include "attention_sweep.h"
 #include "kernels.h"
 
 namespace aeris {
@@ -231,7 +232,21 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
 
   const bool my = p.use_mask && p.sy > 0 && wy == p.nWy - 1;
   const bool mx = p.use_mask && p.sx > 0 && wx == p.nWx - 1;
-  constexpr float MASK_NEG = -100.0f * LOG2E;  // the additive -100 of the shift mask, in the exp2 domain
+  auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(kb * 32 + l31, s2 * 2 + hi));
+  };
+  // V^T fragment of PV step `step` (16 keys): k slots 0-3 <-> keys 16 step + 4hi + (0..3), slots 4-7 <-> keys
+  // 16 step + 8 + 4hi + (0..3): one 16-byte chunk per 32-row block of O^T
+  auto read_v = [&](int step, bf16x8 (&f)[DB]) {
+    const int chunk = step * 2 + hi;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int d = db * 32 + l31;
+      f[db] = *reinterpret_cast<const bf16x8*>(sV + d * VROW + ((chunk ^ v_swz<Cfg::V_SWZ>(d)) << 4));
+    }
+  };
+  const LoadVPlain<DB, decltype(read_v)> load_v(read_v);
 
 #pragma unroll
   for (int ps = 0; ps < 2; ++ps) {
@@ -240,208 +255,14 @@ window_attention_kernel(AttnParams p) {  // at least 2 waves per SIMD: two workg
     int qpos = qg * 32 + l31;
     const bool q_valid = qpos < L;
     if (!q_valid) qpos = L - 1;
-    const int qiy = qpos / WS_X, qix = qpos % WS_X;
-    const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
-    const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
-    const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
-
-    // S^T block kb = K[32 kb ..] Q^T (+ bias): the accumulators start at the relative-position bias (read from LDS
-    // straight into them), so that it costs neither an add nor a zero-fill.
-    // a[4g+i] = logit * log2(e) of key 32 kb + 8 g + 4 hi + i and query qpos.
-    auto init_acc = [&](int kb, f32x16& a) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
-        if (HAS_BIAS) {
-          const int key0 = kb * 32 + g * 8 + hi * 4;
-          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
-          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
-          bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) a[g * 4 + i] = bv[i];
-      }
-    };
-    auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
-#pragma unroll
-      for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<HD>(kb * 32 + l31, s2 * 2 + hi));
-    };
-    // cyclic-shift mask (only windows touching the wrapped border carry more than one region) and the padding keys
-    // of windows whose token count is not a multiple of 32
-    auto mask_block = [&](int kb, f32x16& a) {
-      if (my || mx) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int key = kb * 32 + g * 8 + hi * 4 + i;
-            const int kiy = key / WS_X, kix = key % WS_X;
-            const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
-            const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
-            if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
-          }
-      }
-      if (LPAD != L) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-          if (kb * 32 + g * 8 + hi * 4 >= L) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[g * 4 + i] = -INFINITY;
-          }
-      }
-    };
-    // V^T fragment of PV step `step` (16 keys): k slots 0-3 <-> keys 16 step + 4hi + (0..3), slots 4-7 <-> keys
-    // 16 step + 8 + 4hi + (0..3): one 16-byte chunk per 32-row block of O^T
-    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
-      const int chunk = step * 2 + hi;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int d = db * 32 + l31;
-        f[db] = *reinterpret_cast<const bf16x8*>(sV + d * VROW + ((chunk ^ v_swz<Cfg::V_SWZ>(d)) << 4));
-      }
-    };
-
+    const WindowLogits<WS_Y, WS_X, HAS_BIAS> logits(sB, qpos, hi, my, mx, p.sy, p.sx);
     f32x16 o[DB];
     float sum;
-
-    // ---- fast path: one sweep over the key blocks, P = exp2(logit) without subtracting the row maximum.
-    // softmax is invariant to the subtraction; it only guards the range, and the range is checked afterwards: a row
-    // sum outside [2^-40, 2^100] (or not finite) sends the wave to the two-pass form below.  Per key block the MFMAs
-    // of S^T for block kb + 1 are issued ahead of the exp2 of block kb, and those of P V for block kb after it: the
-    // matrix pipe runs while the VALU forms P.
-    {
-      f32x16 acc3[3];
-      bf16x8 kf[2][KS], vf[2][DB];
-      uint32_t pk[8];
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-      sum = 0.f;
-      load_k(0, kf[0]);
-      init_acc(0, acc3[0]);
-      if (NQ > 1) {
-        load_k(1, kf[1]);
-        init_acc(1, acc3[1]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int s2 = 0; s2 < KS; ++s2)
-        acc3[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0][s2], qf[ps][s2], acc3[0], 0, 0, 0);
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb) {
-        f32x16& a = acc3[kb % 3];
-        __builtin_amdgcn_sched_barrier(0);
-        // LDS reads of this iteration: V^T fragments of the two PV steps of block kb; K fragments and bias of block kb + 2
-        load_v(2 * kb, vf[0]);
-        load_v(2 * kb + 1, vf[1]);
-        if (kb + 1 < NQ) {
-#pragma unroll
-          for (int s2 = 0; s2 < KS; ++s2)
-            acc3[(kb + 1) % 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[(kb + 1) & 1][s2], qf[ps][s2], acc3[(kb + 1) % 3], 0, 0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (kb + 2 < NQ) {
-          load_k(kb + 2, kf[kb & 1]);
-          init_acc(kb + 2, acc3[(kb + 2) % 3]);
-        }
-        mask_block(kb, a);
-#pragma unroll
-        for (int h = 0; h < 8; ++h) {
-          const float e0 = __builtin_amdgcn_exp2f(a[2 * h]);
-          const float e1 = __builtin_amdgcn_exp2f(a[2 * h + 1]);
-          pk[h] = pack_bf16x2(e0, e1);
-          sum = dot2_ones(pk[h], sum);  // the row sum of what PV multiplies: the rounded values
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-          const u32x4 pw = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
-          const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-          for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t2][db], pf, o[db], 0, 0, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      sum += __shfl_xor(sum, 32, 64);
-    }
-    const bool in_range = sum >= 0x1p-40f && sum <= 0x1p100f;  // false for NaN as well
-    if (__builtin_amdgcn_ballot_w64(!in_range) != 0) {
-      // ---- two-pass form for rows whose logits leave the range: all of S^T, row maximum, P = exp2(logit - max)
-      f32x16 acc[NQ];
-      bf16x8 kf[2][KS];
-      load_k(0, kf[0]);
-      init_acc(0, acc[0]);
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb) {
-        if (kb + 1 < NQ) {
-          load_k(kb + 1, kf[(kb + 1) & 1]);
-          init_acc(kb + 1, acc[kb + 1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s2 = 0; s2 < KS; ++s2)
-          acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb & 1][s2], qf[ps][s2], acc[kb], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      float mrow = -INFINITY;
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb) {
-        mask_block(kb, acc[kb]);
-#pragma unroll
-        for (int e = 0; e < 16; e += 2) mrow = fmaxf(fmaxf(mrow, acc[kb][e]), acc[kb][e + 1]);
-      }
-      mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
-      sum = 0.f;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-#pragma unroll
-      for (int step = 0; step < 2 * NQ; ++step) {
-        const int kb = step >> 1, t2 = step & 1;
-        bf16x8 vf[DB];
-        load_v(step, vf);
-        uint32_t pk[4];
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          const int h2 = 4 * t2 + h;
-          const float e0 = __builtin_amdgcn_exp2f(acc[kb][2 * h2] - mrow);
-          const float e1 = __builtin_amdgcn_exp2f(acc[kb][2 * h2 + 1] - mrow);
-          pk[h] = pack_bf16x2(e0, e1);
-          sum = dot2_ones(pk[h], sum);
-        }
-        const u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
-        const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf, o[db], 0, 0, 0);
-      }
-      sum += __shfl_xor(sum, 32, 64);
-    }
-    const float inv = __builtin_amdgcn_rcpf(sum);
-
-    // ---- normalise and store: o[db][4g+i] = O[query][32db + 8g + 4hi + i].  The two lanes of a query (l31 and
-    // l31 + 32) each hold half of every 16-byte piece of the row; v_permlane32_swap on the pieces 2m and 2m + 1
-    // gives the lower lane all of piece 2m and the upper lane all of piece 2m + 1: half as many store
-    // instructions, and 32 contiguous bytes per row and instruction instead of 16.
-    {
-      uint16_t* op = p.out + (uint64_t)q_tok[ps] * (uint32_t)inner + head * HD + hi * 8;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          const int g0 = 2 * m, g1 = 2 * m + 1;
-          const uint32_t x0 = pack_bf16x2(o[db][g0 * 4] * inv, o[db][g0 * 4 + 1] * inv);
-          const uint32_t x1 = pack_bf16x2(o[db][g0 * 4 + 2] * inv, o[db][g0 * 4 + 3] * inv);
-          const uint32_t y0 = pack_bf16x2(o[db][g1 * 4] * inv, o[db][g1 * 4 + 1] * inv);
-          const uint32_t y1 = pack_bf16x2(o[db][g1 * 4 + 2] * inv, o[db][g1 * 4 + 3] * inv);
-          const auto rx = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-          const auto ry = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-          if (q_valid) *reinterpret_cast<u32x4*>(op + db * 32 + m * 16) = u32x4{rx[0], ry[0], rx[1], ry[1]};
-        }
-    }
+    attention_sweep<NQ, KS, DB, HAS_BIAS>(logits, load_k, load_v, [](int) {}, qf[ps], o, sum);
+    store_attention_rows<DB>(p.out + (uint64_t)q_tok[ps] * (uint32_t)inner + head * HD + hi * 8, o, sum, q_valid);
   }
 }
+
 
 // ---------------------------------------------------------------------------------------------
 // The same computation for head_dim 64 with K and V brought into LDS by the load unit itself
@@ -547,25 +368,7 @@ window_attention_dma_kernel(AttnParams p) {
   }
 
   // ---- bias column of this head -> LDS as fp32 4-vectors R4[s] = R[s..s+3] (R reversed, times log2 e)
-  if (HAS_BIAS) {
-    constexpr int BIT = (TBL + NT - 1) / NT;
-    float breg[BIT];
-#pragma unroll
-    for (int it = 0; it < BIT; ++it) {
-      const int j = tid + it * NT;
-      breg[it] = j < TBL ? bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E : 0.f;
-    }
-    float* sBf = reinterpret_cast<float*>(sB);
-#pragma unroll
-    for (int it = 0; it < BIT; ++it) {
-      const int j = tid + it * NT;
-      if (j < TBL) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (j - e >= 0) sBf[(j - e) * 4 + e] = breg[it];
-      }
-    }
-  }
+  if (HAS_BIAS) build_bias_lds<TBL>(sB, p.table, p.heads, head, tid, NT);
   // ---- q * scale * log2(e): the accumulators of K Q^T are then the logits in the exp2 domain
   if (!p.q_prescaled) {
     const float c = p.scale * LOG2E;
@@ -584,19 +387,14 @@ window_attention_dma_kernel(AttnParams p) {
 
   const bool my = p.use_mask && p.sy > 0 && wy == p.nWy - 1;
   const bool mx = p.use_mask && p.sx > 0 && wx == p.nWx - 1;
-  constexpr float MASK_NEG = -100.0f * LOG2E;
 
-  // per-lane part of the V^T fragment addresses: block of 16 lanes jb = lane >> 4 (column half jb & 1, key half hi = jb >> 1),
-  // source lane 4 e + a inside it
-  uint32_t v_lane[DB];
-  {
-    const int jb = lane >> 4, e = (lane >> 2) & 3, a = lane & 3;
+  auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int chunk = (4 * db + 2 * (jb & 1) + (a >> 1)) ^ (2 * e);
-      v_lane[db] = (uint32_t)((4 * (jb >> 1) + e) * 128 + (chunk << 4) + (a & 1) * 8);
-    }
-  }
+    for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<64>(kb * 32 + l31, s2 * 2 + hi));
+  };
+  const uint32_t v_addr = lds_byte_address(sV);
+  auto v_step = [&](int step) { return v_addr + (uint32_t)step * 2048u; };
+  const LoadVTransposed<DB, decltype(v_step)> load_v(lane, v_step);
 
 #pragma unroll
   for (int ps = 0; ps < 2; ++ps) {
@@ -605,183 +403,11 @@ window_attention_dma_kernel(AttnParams p) {
     int qpos = qg * 32 + l31;
     const bool q_valid = qpos < L;
     if (!q_valid) qpos = L - 1;
-    const int qiy = qpos / WS_X, qix = qpos % WS_X;
-    const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
-    const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
-    const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
-
-    auto init_acc = [&](int kb, f32x16& a) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
-        if (HAS_BIAS) {
-          const int key0 = kb * 32 + g * 8 + hi * 4;
-          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
-          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
-          bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) a[g * 4 + i] = bv[i];
-      }
-    };
-    auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
-#pragma unroll
-      for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<64>(kb * 32 + l31, s2 * 2 + hi));
-    };
-    auto mask_block = [&](int kb, f32x16& a) {
-      if (my || mx) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int key = kb * 32 + g * 8 + hi * 4 + i;
-            const int kiy = key / WS_X, kix = key % WS_X;
-            const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
-            const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
-            if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
-          }
-      }
-      if (LPAD != L) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-          if (kb * 32 + g * 8 + hi * 4 >= L) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[g * 4 + i] = -INFINITY;
-          }
-      }
-    };
-    // V^T fragment of PV step `step`: k slots 0-3 <-> keys 16 step + 4 hi + (0..3), slots 4-7 <-> keys 16 step + 8 + 4 hi + (0..3)
-    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048));
-        const bf16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048 + 1024));
-        f[db] = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
-      }
-    };
-
+    const WindowLogits<WS_Y, WS_X, HAS_BIAS> logits(sB, qpos, hi, my, mx, p.sy, p.sx);
     f32x16 o[DB];
     float sum;
-    {  // ---- one sweep over the key blocks, P = exp2(logit), range checked afterwards (see window_attention_kernel)
-      f32x16 acc3[3];
-      bf16x8 kf[2][KS], vf[2][DB];
-      uint32_t pk[8];
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-      sum = 0.f;
-      load_k(0, kf[0]);
-      init_acc(0, acc3[0]);
-      if (NQ > 1) {
-        load_k(1, kf[1]);
-        init_acc(1, acc3[1]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int s2 = 0; s2 < KS; ++s2)
-        acc3[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0][s2], qf[ps][s2], acc3[0], 0, 0, 0);
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb) {
-        f32x16& a = acc3[kb % 3];
-        __builtin_amdgcn_sched_barrier(0);
-        load_v(2 * kb, vf[0]);
-        load_v(2 * kb + 1, vf[1]);
-        if (kb + 1 < NQ) {
-#pragma unroll
-          for (int s2 = 0; s2 < KS; ++s2)
-            acc3[(kb + 1) % 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[(kb + 1) & 1][s2], qf[ps][s2], acc3[(kb + 1) % 3], 0, 0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (kb + 2 < NQ) {
-          load_k(kb + 2, kf[kb & 1]);
-          init_acc(kb + 2, acc3[(kb + 2) % 3]);
-        }
-        mask_block(kb, a);
-#pragma unroll
-        for (int h = 0; h < 8; ++h) {
-          const float e0 = __builtin_amdgcn_exp2f(a[2 * h]);
-          const float e1 = __builtin_amdgcn_exp2f(a[2 * h + 1]);
-          pk[h] = pack_bf16x2(e0, e1);
-          sum = dot2_ones(pk[h], sum);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-          const u32x4 pw = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
-          const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-          for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t2][db], pf, o[db], 0, 0, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      sum += __shfl_xor(sum, 32, 64);
-    }
-    const bool in_range = sum >= 0x1p-40f && sum <= 0x1p100f;
-    if (__builtin_amdgcn_ballot_w64(!in_range) != 0) {
-      // ---- rows whose logits leave the range: row maximum first (S^T recomputed block by block), then P = exp2(logit - max)
-      float mrow = -INFINITY;
-#pragma unroll 1
-      for (int pass = 0; pass < 2; ++pass) {
-        if (pass == 1) {
-          mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
-          sum = 0.f;
-#pragma unroll
-          for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-        }
-#pragma unroll 1
-        for (int kb = 0; kb < NQ; ++kb) {
-          f32x16 a;
-          bf16x8 kf[KS];
-          load_k(kb, kf);
-          init_acc(kb, a);
-#pragma unroll
-          for (int s2 = 0; s2 < KS; ++s2) a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s2], qf[ps][s2], a, 0, 0, 0);
-          mask_block(kb, a);
-          if (pass == 0) {
-#pragma unroll
-            for (int e = 0; e < 16; e += 2) mrow = fmaxf(fmaxf(mrow, a[e]), a[e + 1]);
-          } else {
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-              bf16x8 vf[DB];
-              load_v(2 * kb + t2, vf);
-              uint32_t pk[4];
-#pragma unroll
-              for (int h = 0; h < 4; ++h) {
-                const int h2 = 4 * t2 + h;
-                pk[h] = pack_bf16x2(__builtin_amdgcn_exp2f(a[2 * h2] - mrow), __builtin_amdgcn_exp2f(a[2 * h2 + 1] - mrow));
-                sum = dot2_ones(pk[h], sum);
-              }
-              const u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
-              const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-              for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf, o[db], 0, 0, 0);
-            }
-          }
-        }
-      }
-      sum += __shfl_xor(sum, 32, 64);
-    }
-    const float inv = __builtin_amdgcn_rcpf(sum);
-    {
-      uint16_t* op = p.out + (uint64_t)q_tok[ps] * (uint32_t)inner + head * HD + hi * 8;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          const int g0 = 2 * m, g1 = 2 * m + 1;
-          const uint32_t x0 = pack_bf16x2(o[db][g0 * 4] * inv, o[db][g0 * 4 + 1] * inv);
-          const uint32_t x1 = pack_bf16x2(o[db][g0 * 4 + 2] * inv, o[db][g0 * 4 + 3] * inv);
-          const uint32_t y0 = pack_bf16x2(o[db][g1 * 4] * inv, o[db][g1 * 4 + 1] * inv);
-          const uint32_t y1 = pack_bf16x2(o[db][g1 * 4 + 2] * inv, o[db][g1 * 4 + 3] * inv);
-          const auto rx = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-          const auto ry = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-          if (q_valid) *reinterpret_cast<u32x4*>(op + db * 32 + m * 16) = u32x4{rx[0], ry[0], rx[1], ry[1]};
-        }
-    }
+    attention_sweep<NQ, KS, DB, HAS_BIAS>(logits, load_k, load_v, [](int) {}, qf[ps], o, sum);
+    store_attention_rows<DB>(p.out + (uint64_t)q_tok[ps] * (uint32_t)inner + head * HD + hi * 8, o, sum, q_valid);
   }
 }
 
@@ -822,6 +448,7 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   unsigned char* sB = smem + 4 * KVB;
+  const uint32_t smem_addr = lds_byte_address(smem);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -935,31 +562,21 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
     for (int s2 = 0; s2 < KS; ++s2) q[s2] = *reinterpret_cast<const bf16x8*>(qp + s2 * 16);
   };
   auto build_bias = [&](int head) {
-    if (HAS_BIAS) {
-      float* sBf = reinterpret_cast<float*>(sB);
-      for (int j = tid; j < TBL; j += NT) {
-        const float r = bf16_bits_to_f32(p.table[(int64_t)(TBL - 1 - j) * p.heads + head]) * LOG2E;  // R[j]
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (j - e >= 0) sBf[(j - e) * 4 + e] = r;  // R4[j-e][e] = R[j]
-      }
-    }
+    if (HAS_BIAS) build_bias_lds<TBL>(sB, p.table, p.heads, head, tid, NT);
   };
 
-  // per-lane part of the V^T fragment addresses (see window_attention_dma_kernel)
-  uint32_t v_lane[DB];
-  {
-    const int jb = lane >> 4, e = (lane >> 2) & 3, a = lane & 3;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int chunk = (4 * db + 2 * (jb & 1) + (a >> 1)) ^ (2 * e);
-      v_lane[db] = (uint32_t)((4 * (jb >> 1) + e) * 128 + (chunk << 4) + (a & 1) * 8);
-    }
-  }
-  const int sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
   const float cq = p.scale * LOG2E;
   constexpr float MASK_NEG = -100.0f * LOG2E;
 
+  // A load instruction holds its wave until the CU's one address unit has taken its 64 addresses, and with all waves
+  // issuing their share of the next unit together right after the barrier nothing computes meanwhile.  The upper half
+  // of the waves (the SIMD partners of the lower half) therefore issues its share STAGGER_KB key blocks into the unit:
+  // while one wave of a SIMD queues loads, the other one computes.
+#ifndef AERIS_ATTN_STAGGER
+#define AERIS_ATTN_STAGGER (NQ >= 4 ? NQ / 2 : 0)
+#endif
+  constexpr int STAGGER_KB = AERIS_ATTN_STAGGER;
+  const bool late_issuer = STAGGER_KB > 0 && wave >= NQ / 2;
   Unit cur = decode(u_begin);
   int bias_head = cur.head;
   bf16x8 q_cur[KS], q_nxt[KS];
@@ -992,8 +609,10 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
     if (more) {  // Q first: a later wait for it then does not have to wait for the K / V loads behind it
       load_q(nxt, q_nxt, tok_nxt);
       kv_prepare(nxt);
+      if (!late_issuer) {
 #pragma unroll
-      for (int i = 0; i < N_DMA; ++i) kv_issue(i, set ^ 1);
+        for (int i = 0; i < N_DMA; ++i) kv_issue(i, set ^ 1);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -1001,8 +620,7 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
     const unsigned char* sV = sK + KVB;
     const bool my = p.use_mask && p.sy > 0 && cur.wy == p.nWy - 1;
     const bool mx = p.use_mask && p.sx > 0 && cur.wx == p.nWx - 1;
-    const int ry_q = my ? (qiy < WS_Y - p.sy ? 1 : 2) : 0;
-    const int rx_q = mx ? (qix < WS_X - p.sx ? 1 : 2) : 0;
+    const WindowLogits<WS_Y, WS_X, HAS_BIAS> logits(sB, qpos, hi, my, mx, p.sy, p.sx);
     bf16x8 qf[KS];
 #pragma unroll
     for (int s2 = 0; s2 < KS; ++s2) qf[s2] = q_cur[s2];
@@ -1015,181 +633,27 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
         qf[s2] = __builtin_bit_cast(bf16x8, w);
       }
     }
-
-    auto init_acc = [&](int kb, f32x16& a) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
-        if (HAS_BIAS) {
-          const int key0 = kb * 32 + g * 8 + hi * 4;
-          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
-          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
-          bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) a[g * 4 + i] = bv[i];
-      }
-    };
     auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
 #pragma unroll
       for (int s2 = 0; s2 < KS; ++s2) f[s2] = *reinterpret_cast<const bf16x8*>(sK + k_off<64>(kb * 32 + l31, s2 * 2 + hi));
     };
-    auto mask_block = [&](int kb, f32x16& a) {
-      if (my || mx) {
+    const uint32_t v_addr = smem_addr + (uint32_t)(set * 2 * KVB + KVB);
+    auto v_step = [&](int step) { return v_addr + (uint32_t)step * 2048u; };
+    const LoadVTransposed<DB, decltype(v_step)> load_v(lane, v_step);
+    auto mid = [&](int kb) {  // the late issuers' share of the next unit's loads, STAGGER_KB key blocks into this unit
+      if (STAGGER_KB > 0 && kb == STAGGER_KB && late_issuer && more) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int key = kb * 32 + g * 8 + hi * 4 + i;
-            const int kiy = key / WS_X, kix = key % WS_X;
-            const int ry_k = my ? (kiy < WS_Y - p.sy ? 1 : 2) : 0;
-            const int rx_k = mx ? (kix < WS_X - p.sx ? 1 : 2) : 0;
-            if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
-          }
-      }
-      if (LPAD != L) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-          if (kb * 32 + g * 8 + hi * 4 >= L) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[g * 4 + i] = -INFINITY;
-          }
+        for (int i = 0; i < N_DMA; ++i) kv_issue(i, set ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
       }
     };
-    auto load_v = [&](int step, bf16x8 (&f)[DB]) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048));
-        const bf16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(sV + v_lane[db] + step * 2048 + 1024));
-        f[db] = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
-      }
-    };
-
     f32x16 o[DB];
     float sum;
-    {
-      // one sweep over the key blocks, P = exp2(logit), range checked afterwards (see window_attention_kernel).  Without
-      // a bias the first MFMA of an S^T block takes a literal zero as its C operand, and so does the first one of O^T:
-      // no accumulator is ever zero-filled by the VALU.
-      const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      f32x16 acc2[2];
-      bf16x8 kf[2][KS], vf[2][DB];
-      uint32_t pk[8];
-      sum = 0.f;
-      auto qk_block = [&](int kb, f32x16& acc, const bf16x8 (&kfr)[KS]) {
-#pragma unroll
-        for (int s2 = 0; s2 < KS; ++s2)
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[s2], qf[s2], (!HAS_BIAS && s2 == 0) ? zero16 : acc, 0, 0, 0);
-      };
-      load_k(0, kf[0]);
-      if (HAS_BIAS) init_acc(0, acc2[0]);
-      if (NQ > 1) {
-        load_k(1, kf[1]);
-        if (HAS_BIAS) init_acc(1, acc2[1]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      qk_block(0, acc2[0], kf[0]);
-#pragma unroll
-      for (int kb = 0; kb < NQ; ++kb) {
-        f32x16& a = acc2[kb & 1];
-        __builtin_amdgcn_sched_barrier(0);
-        load_v(2 * kb, vf[0]);
-        load_v(2 * kb + 1, vf[1]);
-        if (kb + 1 < NQ) qk_block(kb + 1, acc2[(kb + 1) & 1], kf[(kb + 1) & 1]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kb + 2 < NQ) load_k(kb + 2, kf[kb & 1]);
-        mask_block(kb, a);
-#pragma unroll
-        for (int h = 0; h < 8; ++h) {
-          const float e0 = __builtin_amdgcn_exp2f(a[2 * h]);
-          const float e1 = __builtin_amdgcn_exp2f(a[2 * h + 1]);
-          pk[h] = pack_bf16x2(e0, e1);
-          sum = dot2_ones(pk[h], sum);  // the row sum of what PV multiplies: the rounded values
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // the accumulators of block kb are consumed: the bias of block kb + 2 goes straight into them
-        if (HAS_BIAS && kb + 2 < NQ) init_acc(kb + 2, a);
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-          const u32x4 pw = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
-          const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-          for (int db = 0; db < DB; ++db)
-            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t2][db], pf, (kb == 0 && t2 == 0) ? zero16 : o[db], 0, 0, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      sum += __shfl_xor(sum, 32, 64);
-    }
-    const bool in_range = sum >= 0x1p-40f && sum <= 0x1p100f;
-    if (__builtin_amdgcn_ballot_w64(!in_range) != 0) {
-      float mrow = -INFINITY;
-#pragma unroll 1
-      for (int pass = 0; pass < 2; ++pass) {
-        if (pass == 1) {
-          mrow = fmaxf(mrow, __shfl_xor(mrow, 32, 64));
-          sum = 0.f;
-#pragma unroll
-          for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-        }
-#pragma unroll 1
-        for (int kb = 0; kb < NQ; ++kb) {
-          f32x16 a;
-          bf16x8 kf[KS];
-          load_k(kb, kf);
-          init_acc(kb, a);
-#pragma unroll
-          for (int s2 = 0; s2 < KS; ++s2) a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s2], qf[s2], a, 0, 0, 0);
-          mask_block(kb, a);
-          if (pass == 0) {
-#pragma unroll
-            for (int e = 0; e < 16; e += 2) mrow = fmaxf(fmaxf(mrow, a[e]), a[e + 1]);
-          } else {
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-              bf16x8 vf[DB];
-              load_v(2 * kb + t2, vf);
-              uint32_t pk[4];
-#pragma unroll
-              for (int h = 0; h < 4; ++h) {
-                const int h2 = 4 * t2 + h;
-                pk[h] = pack_bf16x2(__builtin_amdgcn_exp2f(a[2 * h2] - mrow), __builtin_amdgcn_exp2f(a[2 * h2 + 1] - mrow));
-                sum = dot2_ones(pk[h], sum);
-              }
-              const u32x4 pw = {pk[0], pk[1], pk[2], pk[3]};
-              const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-              for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf, o[db], 0, 0, 0);
-            }
-          }
-        }
-      }
-      sum += __shfl_xor(sum, 32, 64);
-    }
-    const float inv = __builtin_amdgcn_rcpf(sum);
-    {
-      // Always 4 stores per wave and unit (the wait at the top of the loop counts them); rows past the window store
-      // their (recomputed, identical) last row again.  o[db][4g+i] = O[query][32db + 8g + 4hi + i]: v_permlane32_swap
-      // on the pieces 2m and 2m + 1 gives the lower lane of a query all of piece 2m and the upper lane all of piece
-      // 2m + 1: 32 contiguous bytes per row and instruction.  (64 bytes per row through a further v_permlane16_swap,
-      // and the same for the Q loads, measured no faster.)
-      uint16_t* op = p.out + (uint64_t)tok_cur * (uint32_t)inner + cur.head * HD + hi * 8;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          const int g0 = 2 * m, g1 = 2 * m + 1;
-          const uint32_t x0 = pack_bf16x2(o[db][g0 * 4] * inv, o[db][g0 * 4 + 1] * inv);
-          const uint32_t x1 = pack_bf16x2(o[db][g0 * 4 + 2] * inv, o[db][g0 * 4 + 3] * inv);
-          const uint32_t y0 = pack_bf16x2(o[db][g1 * 4] * inv, o[db][g1 * 4 + 1] * inv);
-          const uint32_t y1 = pack_bf16x2(o[db][g1 * 4 + 2] * inv, o[db][g1 * 4 + 3] * inv);
-          const auto rx = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-          const auto ry = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-          *reinterpret_cast<u32x4*>(op + db * 32 + m * 16) = u32x4{rx[0], ry[0], rx[1], ry[1]};
-        }
-    }
+    attention_sweep<NQ, KS, DB, HAS_BIAS>(logits, load_k, load_v, mid, qf, o, sum);
+    // Always DB * 2 stores per wave and unit (the wait at the top of the loop counts them); rows past the window store
+    // their (recomputed, identical) last row again.  (64 bytes per row and instruction through a further
+    // v_permlane16_swap, and the same for the Q loads, measured no faster.)
+    store_attention_rows<DB>(p.out + (uint64_t)tok_cur * (uint32_t)inner + cur.head * HD + hi * 8, o, sum, true);
     cur = nxt;
     tok_cur = tok_nxt;
 #pragma unroll

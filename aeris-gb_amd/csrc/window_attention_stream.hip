@@ -100,6 +100,7 @@ window_attention_stream_kernel(StreamParams p) {
   constexpr float LOG2E = 1.4426950408889634f;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const uint32_t smem_addr = lds_byte_address(smem);
   int* tok = reinterpret_cast<int*>(smem + Cfg::TBL_OFF);  // token row (inside the image) of every window position
   int* const redo = tok + ((p.ws_y * p.ws_x + 3) & ~3);    // set by a wave whose sums left the range of the fast sweep
 
@@ -360,21 +361,32 @@ window_attention_stream_kernel(StreamParams p) {
 
     // PV step (kb, t2): k slots 0-3 <-> keys 32kb+16t2+4hi+(0..3); slots 4-7 <-> keys 32kb+16t2+8+4hi+(0..3): one V^T
     // chunk per 32-row block of O^T.  The fragments of a step are read one step ahead of its MFMAs.
+    // DMA form: the transposing reads are inline assembly (the builtin form would make the compiler wait for the load
+    // unit's pending loads of the next chunks in front of every one of them, see lds_read_tr16_b64); what they return
+    // becomes usable in v_ready().
     bf16x8 vfb[2][DB];
-    auto load_v = [&](int step, bf16x8 (&f)[DB]) {  // f[db] = V^T rows 32 db + l31, chunk step * 2 + hi: vt_off(), taken apart
+    TrFrag vtr[2][DMA ? DB : 1];
+    auto load_v = [&](int step, int slot) {  // V^T rows 32 db + l31, chunk step * 2 + hi: vt_off(), taken apart
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         if (DMA) {  // keys 16 step + 4 hi + (0..3) and 16 step + 8 + 4 hi + (0..3) of row-major V, transposed by the read
-          const uint32_t a0 = v_tr[db] + u * Cfg::V_BYTES + step * 16 * (HD * 2);
-          const bf16x4_t lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(smem + a0));
-          const bf16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(smem + a0 + 8 * (HD * 2)));
-          f[db] = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+          const uint32_t a0 = smem_addr + v_tr[db] + u * Cfg::V_BYTES + step * 16 * (HD * 2);
+          vtr[slot][DMA ? db : 0].lo = lds_read_tr16_b64<0>(a0);
+          vtr[slot][DMA ? db : 0].hi = lds_read_tr16_b64<8 * (HD * 2)>(a0);
         } else {
-          f[db] = *(__attribute__((address_space(3))) const bf16x8*)(v_lane[HD == 128 ? step ^ db : step] + u * Cfg::V_BYTES + db * 4096);
+          vfb[slot][db] = *(__attribute__((address_space(3))) const bf16x8*)(v_lane[HD == 128 ? step ^ db : step] + u * Cfg::V_BYTES + db * 4096);
         }
       }
     };
-    load_v(0, vfb[0]);  // in flight during the softmax arithmetic below
+    auto v_ready = [&](int slot) {
+      if (DMA) {
+        static_assert(!DMA || DB == 4, "the DMA form is built for head_dim 128");
+        lds_tr_wait(vtr[slot][0], vtr[slot][DMA ? 1 : 0], vtr[slot][DMA ? 2 : 0], vtr[slot][DMA ? 3 : 0]);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vfb[slot][db] = tr_frag_value(vtr[slot][DMA ? db : 0]);
+      }
+    };
+    load_v(0, 0);  // in flight during the softmax arithmetic below
 
     // ---- online softmax (exp2 domain): new row max, rescale what has been accumulated if any max moved
     if (!FAST) {
@@ -414,8 +426,9 @@ window_attention_stream_kernel(StreamParams p) {
 #pragma unroll
     for (int step = 0; step < 4; ++step) {
       __builtin_amdgcn_sched_barrier(0);
+      v_ready(step & 1);  // ahead of the next step's reads: the wait then covers reads issued a whole step ago only
       if (step + 1 < 4) {
-        load_v(step + 1, vfb[(step + 1) & 1]);
+        load_v(step + 1, (step + 1) & 1);
         exp_step(step + 1, pkb[(step + 1) & 1]);
       }
       const uint32_t* pk = pkb[step & 1];

@@ -165,6 +165,12 @@ class RoPE2D(nn.Module):
         raise NotImplementedError("RoPE2D is not on the executed path of the reference")
 
 
+# Whether ``Attention`` runs the to_qkv projection inside the attention kernel where that kernel exists (16x16 windows,
+# head_dim 64, dim % 128 == 0) instead of as a GEMM that writes q, k, v to HBM for a separate attention kernel.  Both
+# paths compute the same bits; this picks the faster one as measured on the benchmark's shape.
+FUSE_QKV_ATTENTION = False
+
+
 class Attention(nn.Module):
     """Windowed multi-head self-attention: to_qkv GEMM -> fused window attention -> wo GEMM
     (model.py:265-309).  ``forward(x, shift=(sy, sx))`` folds a cyclic shift into the kernel."""
@@ -178,6 +184,8 @@ class Attention(nn.Module):
         self.window_size, self.image_shape = _pair(window_size), _pair(image_shape)
         self.scale = head_dim ** -0.5
         self.shift_mask = shift_mask
+        self.fuse_qkv = FUSE_QKV_ATTENTION  # per module; see FUSE_QKV_ATTENTION
+        self._b4cache = None
         inner = heads * head_dim
         self.rope = RoPE2D(**{k: v for k, v in rope_kwargs.items() if k in ("window_size", "rope_dim", "rope_base")})
         self.to_qkv = nn.Linear(dim, inner * 3, bias=bias)
@@ -189,9 +197,26 @@ class Attention(nn.Module):
         else:
             self.relative_position_bias_table = None
 
+    def _bias4(self):
+        """The bias table in the fused kernel's form, refreshed whenever the parameter changes."""
+        t = self.relative_position_bias_table
+        if t is None:
+            return None
+        key = (t.data_ptr(), t._version, t.device, t.dtype)
+        if self._b4cache is None or self._b4cache[0] != key:
+            self._b4cache = (key, ops.qkv_attention_pack_bias(t.detach().to(torch.bfloat16).contiguous(), self.window_size))
+        return self._b4cache[1]
+
     def core(self, y, shift=(0, 0), out=None):
         """y bf16 [b, n, d] -> attention output before ``wo`` (bf16 [b*n, inner])."""
         b, n, _ = y.shape
+        use_mask = self.shift_mask and (shift[0] > 0 or shift[1] > 0)
+        if self.fuse_qkv and ops.qkv_attention_supported(y.shape[-1], self.heads, self.head_dim, self.window_size,
+                                                         self.image_shape):
+            # projection and attention in one kernel: q, k, v stay on the chip (same arithmetic, bit-identical result)
+            return ops.qkv_window_attention(y.reshape(b * n, -1), self.to_qkv.weight, self.to_qkv.bias, self._bias4(), b,
+                                            self.image_shape, self.heads, self.head_dim, self.window_size, shift, use_mask,
+                                            self.scale, out=out)
         # q, k, v leave the GEMM as one [b*n, head_dim] plane per part and head (the "(c h d) -> c h d" split of
         # model.py:300 done by the store addresses): a window's rows are then contiguous runs for the attention kernel.
         # The q planes leave the GEMM multiplied by scale * log2(e) in fp32 (model.py:290's `q * self.scale`, in the
@@ -200,8 +225,7 @@ class Attention(nn.Module):
                              out=ops.workspace("qkv", (3 * self.heads, b * n, self.head_dim), torch.bfloat16, y.device),
                              q_scale=self.scale * ops.LOG2E, q_planes=self.heads)
         return ops.window_attention(qkv, b, self.image_shape, self.heads, self.head_dim,
-                                    self.window_size, shift, self.relative_position_bias_table,
-                                    self.shift_mask and (shift[0] > 0 or shift[1] > 0), self.scale, out=out,
+                                    self.window_size, shift, self.relative_position_bias_table, use_mask, self.scale, out=out,
                                     head_planes=True, q_prescaled=True)
 
     def forward(self, x, shift=(0, 0)):
@@ -211,11 +235,27 @@ class Attention(nn.Module):
 
 
 class ModulationLinear(nn.Module):
-    """Linear -> SiLU -> Linear on the noise-level embedding (model.py:311-325); f32 in, f32 out."""
+    """Linear -> SiLU -> Linear on the noise-level embedding (model.py:311-325); f32 in, f32 out.
+
+    Its parameters stay float32 whatever the enclosing module is cast to (``.to(torch.bfloat16)`` moves them and leaves
+    their precision alone).  The shift / scale / gate vectors it produces apply to every token alike, so an error in
+    them is not averaged out over tokens or channels: with these 7 d^2 weights per block rounded to bf16 (what the
+    reference's bf16 layers hold) the residual stream of a 24-block model with O(1) branch gains is off by 5e-3 from
+    this source alone, more than from all four block GEMMs' bf16 weights together.  A bf16 checkpoint loads into them
+    without loss; the two matrix-vector products read 66 MB per block and call instead of 33 MB.
+    """
 
     def __init__(self, dim, out_dim, bias):
         super().__init__()
         self.modulation = nn.Sequential(nn.Linear(dim, dim, bias=bias), nn.SiLU(), nn.Linear(dim, out_dim, bias=bias))
+
+    def _apply(self, fn, recurse=True):
+        def keep_f32(t):
+            r = fn(t)
+            if t.dtype == torch.float32 and r.is_floating_point() and r.dtype != torch.float32:
+                r = t.to(device=r.device)  # follow a move to another device, not a down-cast
+            return r
+        return super()._apply(keep_f32, recurse)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         l0, l2 = self.modulation[0], self.modulation[2]

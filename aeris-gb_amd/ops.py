@@ -184,6 +184,59 @@ def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], he
     return out
 
 
+def qkv_attention_supported(K: int, heads: int, head_dim: int, window_size, image_shape) -> bool:
+    """Whether the fused to_qkv + window attention kernel takes this shape (16x16 windows, head_dim 64, K % 128 == 0)."""
+    H, W = image_shape
+    return (tuple(window_size) == (16, 16) and head_dim == 64 and K % 128 == 0 and H % 16 == 0 and W % 16 == 0
+            and H * W * K * 2 < 0xFFFFFFF0 and 3 * heads * head_dim * K * 2 < 2 ** 31)
+
+
+def qkv_attention_pack_bias(table: torch.Tensor, window_size) -> torch.Tensor:
+    """The relative-position bias table [(2ws-1)^2, heads] bf16 in the form ``qkv_window_attention`` reads."""
+    _dev(table, "bias_table", torch.bfloat16)
+    heads = table.shape[1]
+    n = int(L.lib().aeris_qkv_attention_bias_bytes(heads, window_size[0], window_size[1]))
+    if n <= 0 or table.shape[0] != (2 * window_size[0] - 1) * (2 * window_size[1] - 1):
+        raise RuntimeError(f"no fused kernel for windows {tuple(window_size)} / table {tuple(table.shape)}")
+    out = torch.empty(n // 4, dtype=torch.float32, device=table.device)
+    L.call("aeris_qkv_attention_prepare_bias", table.data_ptr(), heads, window_size[0], window_size[1], out.data_ptr(), _stream())
+    return out
+
+
+def qkv_window_attention(y: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], bias4: Optional[torch.Tensor], B: int,
+                         image_shape: Tuple[int, int], heads: int, head_dim: int, window_size: Tuple[int, int],
+                         shift: Tuple[int, int] = (0, 0), use_mask: bool = False, scale: Optional[float] = None,
+                         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y bf16 [B*H*W, K] -> attention output bf16 [B*H*W, heads*head_dim] with the to_qkv projection (w [3*inner, K],
+    bias [3*inner] | None) inside the kernel; ``bias4`` from ``qkv_attention_pack_bias`` (None: no rel-pos bias)."""
+    H, W = image_shape
+    inner = heads * head_dim
+    _dev(y, "y", torch.bfloat16)
+    _dev(w, "w", torch.bfloat16)
+    K = y.shape[-1]
+    if y.numel() != B * H * W * K or tuple(w.shape) != (3 * inner, K):
+        raise RuntimeError(f"y must hold {B}*{H}*{W} rows of {K}, w must be [{3 * inner}, {K}]")
+    if bias is not None:
+        _dev(bias, "bias", torch.bfloat16)
+        if bias.numel() != 3 * inner:
+            raise RuntimeError("bias has the wrong size")
+    if bias4 is not None:
+        _dev(bias4, "bias4", torch.float32)
+    if out is None:
+        out = torch.empty(B * H * W, inner, dtype=torch.bfloat16, device=y.device)
+    else:
+        _dev(out, "out", torch.bfloat16)
+        if out.numel() != B * H * W * inner:
+            raise RuntimeError("out has the wrong size")
+    Lw = window_size[0] * window_size[1]
+    S = B * H * W
+    with _timed("qkv_window_attention", 2.0 * S * 3 * inner * K + 4.0 * S * Lw * inner, "flop"):
+        L.call("aeris_qkv_window_attention_fwd", y.data_ptr(), w.data_ptr(), _ptr(bias), _ptr(bias4), out.data_ptr(), B, H, W,
+               heads, head_dim, K, window_size[0], window_size[1], shift[0], shift[1], int(bool(use_mask)),
+               float(head_dim ** -0.5 if scale is None else scale), _stream())
+    return out
+
+
 def _rowvec(t: Optional[torch.Tensor], name: str, d: int, B: int):
     """f32 [1|B, d] row vectors, rows possibly strided (a chunk of a wider matrix): -> (ptr, batch stride)."""
     if t is None:

@@ -102,6 +102,25 @@ int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const vo
                                      int heads, int head_dim, int ws_y, int ws_x, int shift_y, int shift_x,
                                      int use_mask, float scale, int q_prescaled, int64_t plane_stride, void* stream);
 
+/* to_qkv projection and window attention in one kernel: q, k and v never leave the chip.
+ *   y    bf16 [B*H*W, K]      the normalised tokens, natural (row-major lat x lon) order
+ *   w    bf16 [3*heads*head_dim, K], rows ordered (c h d) like to_qkv.weight (model.py:284,300); qkv_bias bf16
+ *        [3*heads*head_dim] or NULL
+ *   bias4  the relative-position bias table in the form aeris_qkv_attention_prepare_bias writes
+ *        (aeris_qkv_attention_bias_bytes(heads, ws_y, ws_x) bytes, to be refreshed when the table changes), or NULL
+ *   out  bf16 [B*H*W, heads*head_dim]
+ * One (window, head) at a time: the window's rows of y (gathered through the folded partition / shift index map) times
+ * the head's 3*head_dim weight rows, bias added and q multiplied by scale * log2(e) in fp32, one rounding to bf16, then
+ * the same softmax(q k^T + bias + mask) v as aeris_window_attention_heads_fwd from on-chip memory.  Replaces
+ * model.py:299-307 (+ the swin_shift calls at model.py:471-475 on one device): the same result as aeris_gemm_heads_fwd
+ * (with q_scale) followed by aeris_window_attention_heads_fwd (q_prescaled), bit for bit.
+ * Built for 16x16 windows, head_dim 64, K % 128 == 0, H*W*K*2 < 2^32; anything else: AERIS_EUNSUPPORTED. */
+int64_t aeris_qkv_attention_bias_bytes(int heads, int ws_y, int ws_x);
+int aeris_qkv_attention_prepare_bias(const void* bias_table, int heads, int ws_y, int ws_x, void* out, void* stream);
+int aeris_qkv_window_attention_fwd(const void* y, const void* w, const void* qkv_bias, const void* bias4, void* out,
+                                   int B, int H, int W, int heads, int head_dim, int K, int ws_y, int ws_x,
+                                   int shift_y, int shift_x, int use_mask, float scale, void* stream);
+
 /* Row norm fused with noise-level modulation.
  *   x  [B*rows_per_batch, d] (x_dtype bf16|f32)  ->  y [B*rows_per_batch, d] (y_dtype bf16|f32)
  *   gamma [d]; beta [d] or NULL (both param_dtype bf16|f32); shift, scale f32 [B_mod, d] or NULL

@@ -382,6 +382,68 @@ def test_gemm_heads_scales_the_query_planes_in_fp32(pkg, cuda, shape):
             assert rel_l2(got.cpu(), ref.cpu()) <= 2.5e-3  # one bf16 rounding: 2^-9 / sqrt(3) = 1.1e-3 on average
 
 
+FUSED_CASES = [
+    # B, H, W, heads, K, shift, bias + mask, projection bias -- 16x16 windows, head_dim 64: the fused to_qkv + attention kernel
+    (1, 160, 160, 24, 1536, 8, True, True),    # configs[3] widths: 24 k-tiles, 2400 units
+    (1, 160, 160, 24, 256, 0, False, False),   # 4 k-tiles, no bias anywhere: accumulators start at a literal zero
+    (2, 96, 160, 6, 384, 8, True, False),      # two batch entries, 120 windows x 6 heads
+    (1, 48, 80, 3, 128, 8, True, True),        # 15 windows (the last group of 4 is short), 2 k-tiles, 45 units < 256 workgroups
+    (1, 32, 32, 2, 640, 8, True, True),        # every window on the wrapped border; 8 units
+]
+
+
+@pytest.mark.parametrize("case", FUSED_CASES, ids=lambda c: f"B{c[0]}_{c[1]}x{c[2]}_h{c[3]}_K{c[4]}_s{c[5]}_b{int(c[6])}_pb{int(c[7])}")
+def test_fused_qkv_window_attention(pkg, cuda, case):
+    """The to_qkv projection inside the attention kernel (q, k, v never in HBM) against the two-kernel path (GEMM writing
+    head planes with q scaled in its epilogue, then the attention kernel): the same arithmetic in the same order, so
+    bit-identical wherever the GEMM of the two-kernel path is the 256x256-tile kernel (same MFMA shape and k order), and
+    within the ordinary tolerance of the fp32 oracle everywhere."""
+    B, H, W, heads, K, sh, bias_mask, proj_bias = case
+    hd, ws = 64, 16
+    g = torch.Generator().manual_seed(H * W + heads + K)
+    inner, S = heads * hd, B * H * W
+    y = bf(torch.randn(S, K, generator=g))
+    w = bf(torch.randn(3 * inner, K, generator=g) / math.sqrt(K))
+    pb = bf(0.3 * torch.randn(3 * inner, generator=g)) if proj_bias else None
+    table = bf(0.7 * torch.randn((2 * ws - 1) ** 2, heads, generator=g)) if bias_mask else None
+    ops = pkg.ops
+    assert ops.qkv_attention_supported(K, heads, hd, (ws, ws), (H, W))
+    yd, wd = y.to(cuda), w.to(cuda)
+    pbd = None if pb is None else pb.to(cuda)
+    td = None if table is None else table.to(cuda)
+    b4 = None if td is None else ops.qkv_attention_pack_bias(td, (ws, ws))
+    got = ops.qkv_window_attention(yd, wd, pbd, b4, B, (H, W), heads, hd, (ws, ws), (sh, sh), bias_mask)
+    got2 = ops.qkv_window_attention(yd, wd, pbd, b4, B, (H, W), heads, hd, (ws, ws), (sh, sh), bias_mask)
+    planes = ops.gemm_heads(yd, wd, pbd, hd, q_scale=hd ** -0.5 * LOG2E, q_planes=heads)
+    two = ops.window_attention(planes, B, (H, W), heads, hd, (ws, ws), (sh, sh), td, bias_mask, head_planes=True,
+                               q_prescaled=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got, got2) and bool(torch.isfinite(got.float()).all())
+    if ops.gemm_uses_big_tiles(S, 3 * inner):
+        assert torch.equal(got, two)
+    else:
+        assert rel_l2(got, two) <= 4e-3, rel_l2(got, two)
+    cfg = OracleConfig(dim=inner, heads=heads, head_dim=hd, mlp_dim=inner, window_size=(ws, ws), image_shape=(H, W),
+                       rel_pos_bias=bias_mask, shift_mask=bias_mask)
+    qkv = y.float() @ w.float().T + (0 if pb is None else pb.float())
+    ref = attention_core(cfg, qkv.view(B, H * W, 3 * inner), (sh, sh), None if table is None else table.float())
+    err = rel_l2(got.view(B, H * W, inner), ref)
+    print(f"fused qkv + attention {case}: rel-L2 vs fp32 oracle {err:.3e}")
+    assert err <= 6e-3, err
+
+
+def test_fused_qkv_window_attention_rejects_other_shapes(pkg, cuda):
+    ops = pkg.ops
+    assert not ops.qkv_attention_supported(1536, 24, 64, (12, 12), (180, 360))
+    assert not ops.qkv_attention_supported(1536, 12, 128, (16, 16), (160, 160))
+    assert not ops.qkv_attention_supported(1472, 24, 64, (16, 16), (160, 160))  # K % 128
+    y = torch.zeros(144 * 4, 128, dtype=torch.bfloat16, device=cuda)
+    w = torch.zeros(3 * 64, 128, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(pkg.AerisError) as e:
+        ops.qkv_window_attention(y, w, None, None, 1, (24, 24), 1, 64, (12, 12))
+    assert e.value.code == -2
+
+
 NONFINITE_CASES = [
     # B, H, W, heads, hd, ws, shift, bias + mask, head planes -- one case per kernel form
     ("persistent", 1, 160, 160, 24, 64, 16, 8, True, True),

@@ -118,6 +118,20 @@ def test_argument_validation_needs_no_gpu(pkg):
     assert "q_planes" in L.last_error()
     assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64, 0.0, 1, None) == L.EINVAL  # q_scale must be positive
     assert hh(p16, p16, p16, None, 8, 128, 64, 64, 8 * 64, float("nan"), 1, None) == L.EINVAL
+    # fused to_qkv + window attention
+    qa, qb, qp = lib.aeris_qkv_window_attention_fwd, lib.aeris_qkv_attention_bias_bytes, lib.aeris_qkv_attention_prepare_bias
+    assert qb(24, 16, 16) == 24 * 961 * 16 and qb(24, 12, 12) == 0 and qb(0, 16, 16) == 0
+    assert qp(None, 24, 16, 16, p16, None) == L.EINVAL and qp(p16, 24, 8, 8, p16, None) == L.EUNSUPPORTED
+    okq = (p16, p16, None, None, p16, 1, 32, 32, 2, 64, 128, 16, 16, 8, 8, 1, 0.125, None)
+    def withq(i, v):
+        a = list(okq); a[i] = v; return a
+    assert qa(*withq(0, None)) == L.EINVAL and qa(*withq(4, None)) == L.EINVAL  # y / out NULL
+    assert qa(*withq(2, p16 + 2)) == L.EINVAL  # projection bias not 8-byte aligned
+    assert qa(*withq(9, 128)) == L.EUNSUPPORTED and qa(*withq(10, 192)) == L.EUNSUPPORTED  # head_dim, K % 128
+    assert qa(*withq(11, 32)) == L.EUNSUPPORTED  # 32x16 windows
+    assert "aeris_gemm_heads_fwd" in L.last_error()  # the message names the two-kernel path to use instead
+    assert qa(*withq(13, 16)) == L.EINVAL  # shift outside the window
+    assert qa(*withq(16, 0.0)) == L.EINVAL  # scale
     # fused output stage
     osf, osw = lib.aeris_output_stage_fwd, lib.aeris_output_stage_workspace_bytes
     assert osw(69, 1536, 1) == 1536 * 80 * 4 + 80 * 8 and osw(69, 1536, 4) == 4 * osw(69, 1536, 1)
@@ -195,8 +209,9 @@ def test_ref_state_dict_layout_matches_reference(pkg):
             want.update({p + "0.weight": ((d,), torch.bfloat16), p + "1.to_qkv.weight": ((3 * inner, d), torch.bfloat16),
                          p + "1.wo.weight": ((d, inner), torch.bfloat16), p + "2.weight": ((d,), torch.bfloat16),
                          p + "3.w1.weight": ((2 * Hd, d), torch.bfloat16), p + "3.w2.weight": ((d, Hd), torch.bfloat16),
-                         p + "4.modulation.0.weight": ((d, d), torch.bfloat16), p + "4.modulation.0.bias": ((d,), torch.bfloat16),
-                         p + "4.modulation.2.weight": ((6 * d, d), torch.bfloat16), p + "4.modulation.2.bias": ((6 * d,), torch.bfloat16)})
+                         # the modulation MLP keeps f32 parameters (same keys and shapes; a bf16 checkpoint loads without loss)
+                         p + "4.modulation.0.weight": ((d, d), torch.float32), p + "4.modulation.0.bias": ((d,), torch.float32),
+                         p + "4.modulation.2.weight": ((6 * d, d), torch.float32), p + "4.modulation.2.bias": ((6 * d,), torch.float32)})
     assert set(sd.keys()) == set(want.keys())
     for k, (shape, dt) in want.items():
         assert tuple(sd[k].shape) == shape and sd[k].dtype == dt, k

@@ -188,14 +188,14 @@ int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const vo
 }
 
 int64_t aeris_qkv_attention_bias_bytes(int heads, int ws_y, int ws_x) {
-  if (heads <= 0 || !aeris::qkv_attention_supported(ws_y, ws_x, 64, 128, 1)) return 0;
+  if (heads <= 0 || !aeris::qkv_attention_supported(ws_y, ws_x, 64, 256, 1)) return 0;
   return aeris::qkv_attention_bias_bytes(heads);
 }
 
 int aeris_qkv_attention_prepare_bias(const void* bias_table, int heads, int ws_y, int ws_x, void* out, void* stream) {
   if (!bias_table || !out) return fail(AERIS_EINVAL, "aeris_qkv_attention_prepare_bias: bias_table/out is NULL");
   if (heads <= 0) return fail(AERIS_EINVAL, "aeris_qkv_attention_prepare_bias: heads must be positive");
-  if (!aeris::qkv_attention_supported(ws_y, ws_x, 64, 128, 1))
+  if (!aeris::qkv_attention_supported(ws_y, ws_x, 64, 256, 1))
     return fail(AERIS_EUNSUPPORTED, "aeris_qkv_attention_prepare_bias: only 16x16 windows are built (got %dx%d)", ws_y, ws_x);
   if (!aligned16(out)) return fail(AERIS_EINVAL, "aeris_qkv_attention_prepare_bias: out must be 16-byte aligned");
   hipError_t e = aeris::qkv_attention_bias_launch(bias_table, reinterpret_cast<float*>(out), heads, reinterpret_cast<hipStream_t>(stream));
@@ -216,7 +216,7 @@ int aeris_qkv_window_attention_fwd(const void* y, const void* w, const void* qkv
   if (!(scale > 0.f)) return fail(AERIS_EINVAL, "%s: scale must be positive", who);
   if (!aeris::qkv_attention_supported(ws_y, ws_x, head_dim, K, (int64_t)H * W))
     return fail(AERIS_EUNSUPPORTED,
-                "%s: built for 16x16 windows, head_dim 64, K a multiple of 128 and H*W*K*2 < 2^32 (got %dx%d, head_dim %d, "
+                "%s: built for 16x16 windows, head_dim 64, K a multiple of 128 and at least 256, H*W*K*2 < 2^32 (got %dx%d, head_dim %d, "
                 "K %d, H*W %lld): use aeris_gemm_heads_fwd + aeris_window_attention_heads_fwd", who, ws_y, ws_x, head_dim, K,
                 (long long)H * W);
   if ((int64_t)3 * heads * head_dim * K * 2 >= (int64_t(1) << 31))

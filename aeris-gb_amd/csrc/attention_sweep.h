@@ -192,9 +192,18 @@ __device__ __forceinline__ void attention_sweep(const Logits& lg, const LoadK& l
       f32x16& a = acc2[kb & 1];
       __builtin_amdgcn_sched_barrier(0);
       mid(kb);
+      // S^T of the next block first, the V^T reads of this block behind it: the compiler's wait for the bias vectors
+      // and K fragments that those MFMAs consume (it does not know of the assembly reads and waits for "all") then
+      // falls where only reads issued a block ago are outstanding, not on top of the V^T reads just issued
+      if (kb + 1 < NQ) qk_block(acc2[(kb + 1) & 1], kf[(kb + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
       load_v(2 * kb, vraw[0]);
       load_v(2 * kb + 1, vraw[1]);
-      if (kb + 1 < NQ) qk_block(acc2[(kb + 1) & 1], kf[(kb + 1) & 1]);
+      // Keep every accumulator of the S^T block just issued live across these reads.  Where the compiler can prove part
+      // of it unused (keys past the window become -inf whatever the MFMA wrote) it would hand those registers to the
+      // V^T reads, and it places no wait between an MFMA still writing a register and an assembly read returning into
+      // it: the MFMA's late write would replace the V^T fragment.
+      if (kb + 1 < NQ) asm volatile("" : "+v"(acc2[(kb + 1) & 1]));
       __builtin_amdgcn_sched_barrier(0);
       if (kb + 2 < NQ) load_k(kb + 2, kf[kb & 1]);
       lg.mask_block(kb, a);

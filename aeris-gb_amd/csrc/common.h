@@ -48,6 +48,31 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// ---- buffer_load_dwordx4 ... lds (16 bytes per lane from global memory straight into LDS, lane l at LDS byte
+// m0 + 16 l) as inline assembly.  The compiler's builtin form makes every later LDS access a possible alias of the load
+// in the compiler's eyes: it then guards LDS reads with s_waitcnt vmcnt(0) wherever it cannot count the operations in
+// between, e.g. inside a loop that is entered with stores still in flight.  Issued from assembly the load is invisible
+// to that bookkeeping; what orders it against the LDS reads is the kernels' own counted s_waitcnt + barrier, as
+// before.  (Vector memory operations complete in order, so operations the compiler does not know of only make its own
+// counted waits stricter.)  The descriptor is built by hand: base, stride 0, size in bytes, raw 32-bit format.
+typedef u32x4 lds_dma_rsrc;
+__device__ __forceinline__ lds_dma_rsrc make_lds_dma_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  lds_dma_rsrc r;
+  r.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  r.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+  r.z = __builtin_amdgcn_readfirstlane(bytes);
+  r.w = 0x00020000u;
+  return r;
+}
+// lds_address, soffset: wave-uniform; voffset: per lane; out-of-range lanes (voffset >= size) arrive as zeros
+__device__ __forceinline__ void lds_dma_load16(const lds_dma_rsrc& rsrc, uint32_t lds_address, uint32_t voffset, uint32_t soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_address), "v"(voffset), "s"(rsrc), "s"(soffset)
+               : "memory");
+}
+
 // ---- ds_read_b64_tr_b16 (the LDS read that transposes 4 x 4 blocks of 16-bit elements on the way out) as inline assembly.
 // The compiler's builtin form may not be used while a buffer_load ... lds is in flight: the compiler cannot tell that
 // the read does not alias the load's destination and puts an s_waitcnt vmcnt(0) in front of it, which makes a wave

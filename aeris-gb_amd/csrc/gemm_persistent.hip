@@ -37,10 +37,6 @@ constexpr int A_STAGES = 2, B_STAGES = 3;
 constexpr int B_OFF = A_STAGES * A_BYTES;
 constexpr int SMEM = A_STAGES * A_BYTES + B_STAGES * B_BYTES;  // 160 KB: all of the CU's LDS
 constexpr int GM = 4;                     // row panels per L2 group
-#ifndef AERIS_GEMM_EARLY_BIAS
-#define AERIS_GEMM_EARLY_BIAS 0
-#endif
-constexpr bool EARLY_BIAS = AERIS_GEMM_EARLY_BIAS != 0;
 }  // namespace
 
 // PLAIN: no gate and no residual (qkv, fc1): the epilogue is compiled without those paths - about 2 % faster than
@@ -235,10 +231,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     const int ld24 = (int)p.ldc, rs24 = (int)c_row_stride(p);
     const int rrow_t = rrow;
     const int n_wave = tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);  // first output column of this wave
-    u32x2 bq_next[FN];  // the next tile's bias, for its accumulators
-    // EARLY_BIAS: requested before anything else of the epilogue, so that the wait for it at the end counts the
-    // operations issued after it and does not wait for a single store; otherwise ahead of the last block's stores.
-    if (EARLY_BIAS && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+    u32x2 bq_next[FN];  // loaded ahead of the last block's stores, used after them
     // The query part of a qkv projection is multiplied by q_scale here, in fp32, before its only rounding.  Whole
     // 64-column wave blocks lie inside or outside the query columns (q_cols % 64 == 0, checked at launch): a
     // wave-uniform branch that two thirds of the tiles of such a projection skip.
@@ -352,7 +345,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       }
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
-        if (!EARLY_BIAS && i + 1 == FM && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+        if (i + 1 == FM && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
 #pragma unroll
         for (int m = 0; m < NP; ++m) {
           float a[4], b[4];
@@ -406,7 +399,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_wave_barrier();
         // the next loads go ahead of the stores below
         if (RES_BF16 && i + 2 < FM / 2) load_res(i + 2);
-        if (!EARLY_BIAS && i + 1 == FM / 2 && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+        if (i + 1 == FM / 2 && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
 #pragma unroll
         for (int it = 0; it < 4; ++it)
           *reinterpret_cast<u32x4*>(c_lane + (int64_t)__mul24(i * 32 + rrow + 8 * it, rs24) * 2) = out[it];
@@ -495,7 +488,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_wave_barrier();
         if (i + 1 < FM / 2) {
           if (res_dtype >= 0) load_res(i + 1);  // ahead of the stores below
-        } else if (!EARLY_BIAS && r_done + 1 < n_my) {
+        } else if (r_done + 1 < n_my) {
           load_bias(r_done + 1, bq_next);
         }
 #pragma unroll
@@ -557,7 +550,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (u + 2 < UNITS) load_res(u + 2);  // ahead of the stores below
-        if (!EARLY_BIAS && u + 1 == UNITS && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+        if (u + 1 == UNITS && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
 #pragma unroll
         for (int it = 0; it < 4; ++it)
           *reinterpret_cast<f32x4*>(c_lane + ((int64_t)__mul24(i * 32 + rrow + 8 * it, ld24) + j * 32) * 4) = out[it];
@@ -634,7 +627,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_wave_barrier();
         if (u + 1 < UNITS) {
           if (p.res_dtype >= 0) load_res(u + 1);  // ahead of the stores below
-        } else if (!EARLY_BIAS && r_done + 1 < n_my) {
+        } else if (r_done + 1 < n_my) {
           load_bias(r_done + 1, bq_next);
         }
         const int n = unit_col(u);
@@ -726,7 +719,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     // Nothing that writes a register may be pending when the k-loop is entered: the compiler would guard the
     // fragment registers with a wait for all vector memory operations inside the loop, on every k-tile, which
     // cuts the lead of the W loads to one slot.  The first k-tile needs the oldest loads at once anyway.
-    if (!EARLY_BIAS) __builtin_amdgcn_s_waitcnt(WAIT_VM0);
+    __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   }
 }
 

@@ -21,12 +21,15 @@
 //                 wave has its Q fragments.  K must be even for that (the last k-tile then uses A1).
 //   bias          the head's relative-position bias as fp32 4-vectors (WindowLogits), prepared once per parameter value
 //                 by qkv_attention_bias_kernel, brought in by the load unit during the main loop
-// Units are ordered like the tiles of the persistent GEMM: each XCD owns a contiguous chunk, walked 4 windows x all
-// heads at a time, so that a window's token rows and a head's weight rows are shared in that XCD's L2.
+// Units are walked in groups of 4 windows x all heads, so that a window's token rows and a head's weight rows are
+// shared in one XCD's L2; the groups are dealt to the 8 XCDs in turn (group g to XCD g % 8) and the units of an XCD's
+// groups to its workgroups in turn, which spreads the windows on the wrapped border of a shifted grid - a whole
+// window row, slower than the others by their mask arithmetic - evenly over XCDs and workgroups.
 #include "common.h"
 #include "attention_sweep.h"
 #include "gemm_common.h"
 #include "kernels.h"
+#include <type_traits>
 
 namespace aeris {
 
@@ -59,7 +62,7 @@ struct QkvAttnParams {
   int sy, sx;
   int use_mask;
   float q_scale;          // softmax scale times log2(e)
-  int n_win, total_units, per_xcd, bpx;
+  int n_win, bpx;         // windows (B * nWy * nWx); workgroups per XCD
 };
 }  // namespace
 
@@ -88,18 +91,22 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
   const int H = p.H, W = p.W;
   const int inner = p.heads * QA_HD;
 
-  // ---- this workgroup's unit list (as the tiles of the persistent GEMM: XCD x owns [x * per_xcd, (x + 1) * per_xcd))
+  // ---- this workgroup's unit list: XCD x (workgroup id & 7: consecutive workgroups go to consecutive XCDs) owns the
+  // groups x, x + 8, ...; its workgroup `slot` takes the units slot, slot + bpx, ... of those groups laid end to end.
+  // Only the very last group can be short (fewer than QA_GM windows) and it ends its XCD's sequence.
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int chunk0 = xcd * p.per_xcd;
-  int chunk_len = p.total_units - chunk0;
-  if (chunk_len > p.per_xcd) chunk_len = p.per_xcd;
-  const int n_my = chunk_len > slot ? (chunk_len - slot + p.bpx - 1) / p.bpx : 0;
+  const int gsz = QA_GM * p.heads;
+  const int n_groups = (p.n_win + QA_GM - 1) / QA_GM;
+  const int my_groups = n_groups > xcd ? (n_groups - xcd + 7) / 8 : 0;
+  int seq_len = my_groups * gsz;
+  if (my_groups > 0 && (my_groups - 1) * 8 + xcd == n_groups - 1) seq_len -= (n_groups * QA_GM - p.n_win) * p.heads;
+  const int n_my = seq_len > slot ? (seq_len - slot + p.bpx - 1) / p.bpx : 0;
   if (n_my == 0) return;
   struct Unit { int head, b, wy, wx; };
   auto decode = [&](int r) {
-    const int t = chunk0 + r * p.bpx + slot;
-    const int gsz = QA_GM * p.heads;
-    const int g = t / gsz, within = t - g * gsz;
+    const int t = r * p.bpx + slot;
+    const int lg = t / gsz, within = t - lg * gsz;
+    const int g = lg * 8 + xcd;
     int gm = p.n_win - g * QA_GM;
     if (gm > QA_GM) gm = QA_GM;
     Unit u;
@@ -173,12 +180,22 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
 #pragma unroll
       for (int i = 0; i < 4; ++i) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(sd + i * 1024), 16, la_voff[i], so, 0, 0);
       la_stage ^= 1;
-      if (++la_kt == KT) {
-        la_kt = 0;
-        ++la_r;
-        la_set_unit();
-      }
+      ++la_kt;
     }
+  };
+  auto la_next_unit = [&]() {  // the stream has issued all k-tiles of its unit: on to the next one
+    la_kt = 0;
+    ++la_r;
+    la_set_unit();
+  };
+  // the same inside a unit (k-tiles 1 .. KT - 1 of the unit the stream is in): no end-of-list or end-of-unit decisions
+  auto issue_a_same_unit = [&]() {
+    unsigned char* sd = smem + la_stage * QA_A_BYTES + wave_u * 4096;
+    const uint32_t so = la_base + (uint32_t)la_kt * (QA_BK * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(sd + i * 1024), 16, la_voff[i], so, 0, 0);
+    la_stage ^= 1;
+    ++la_kt;
   };
   int lw_r = 0, lw_kt = 0, lw_stage = 0;  // W stream
   uint32_t lw_row[3];                     // W row of the first row of each of this wave's three 8-row blocks
@@ -199,13 +216,24 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
       for (int i = 0; i < 3; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(sd + i * 1024), 16, w_voff[(wave_u * 3 + i) & 1],
                                                  lw_row[i] * rowb + kb, 0, 0);
-      if (++lw_stage == 3) lw_stage = 0;
-      if (++lw_kt == KT) {
-        lw_kt = 0;
-        ++lw_r;
-        lw_set_unit();
-      }
+      lw_stage = lw_stage == 2 ? 0 : lw_stage + 1;
+      ++lw_kt;
     }
+  };
+  auto lw_next_unit = [&]() {
+    lw_kt = 0;
+    ++lw_r;
+    lw_set_unit();
+  };
+  auto issue_w_same_unit = [&]() {
+    unsigned char* sd = smem + QA_W_OFF + lw_stage * QA_W_BYTES + wave_u * 3072;
+    const uint32_t kb = (uint32_t)lw_kt * (QA_BK * 2);
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(sd + i * 1024), 16, w_voff[(wave_u * 3 + i) & 1],
+                                               lw_row[i] * rowb + kb, 0, 0);
+    lw_stage = lw_stage == 2 ? 0 : lw_stage + 1;
+    ++lw_kt;
   };
   // the head's bias 4-vectors -> LDS: 16 load instructions of 1 KB, two per wave (the last one ends outside the
   // descriptor: zeros)
@@ -270,6 +298,21 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
     const int l15 = lane_t & 15, q4 = lane_t >> 4, l31 = lane_t & 31, hi = lane_t >> 5;
     const int qpos = wave_u * 32 + l31;
     const uint32_t q_rel = (uint32_t)((qpos / QA_WS) * W + qpos % QA_WS);
+#if defined(QA_LAB) && QA_LAB == 2
+    {  // timing only: the main loop alone (the accumulators are folded into one store so that they stay live)
+      f32x4 t = {0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < QA_FM; ++i) for (int j = 0; j < QA_FN; ++j) t += acc[i][j];
+      la_next_unit();
+      issue_a();
+      *reinterpret_cast<f32x4*>(p.out + ((uint64_t)un.b * (uint32_t)(H * W) + window_base(un) + q_rel) * (uint32_t)inner + un.head * QA_HD + hi * 8) = t;
+      u32x2 bq0[QA_FN];
+      for (int j = 0; j < QA_FN; ++j) bq0[j] = u32x2{0u, 0u};
+      init_acc(bq0);
+      __builtin_amdgcn_s_waitcnt(WAIT_ALL);
+      __builtin_amdgcn_s_barrier();
+      return;
+    }
+#endif
     unsigned char* const sQ = smem;                                   // A0: idle, its refill is issued below
     unsigned char* const sK = smem + QA_A_BYTES;                      // A1: the last k-tile's stage
     unsigned char* const sV0 = smem + QA_W_OFF + sw_last * QA_W_BYTES;  // the last k-tile's W stage: V rows 0..191
@@ -311,11 +354,13 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     // every wave has its Q: A0 may be refilled with the next unit's first k-tile (held back in the main loop)
+    la_next_unit();
     issue_a();
     __builtin_amdgcn_sched_barrier(0);
     // 3. the sweep
-    const bool my = p.use_mask && p.sy > 0 && un.wy == p.nWy - 1;
-    const bool mx = p.use_mask && p.sx > 0 && un.wx == p.nWx - 1;
+    // (wave-uniform, and said so: the mask arithmetic must stay behind a scalar branch that all but the border windows skip)
+    const bool my = __builtin_amdgcn_readfirstlane((int)(p.use_mask && p.sy > 0 && un.wy == p.nWy - 1)) != 0;
+    const bool mx = __builtin_amdgcn_readfirstlane((int)(p.use_mask && p.sx > 0 && un.wx == p.nWx - 1)) != 0;
     const WindowLogits<QA_WS, QA_WS, HAS_BIAS> logits(smem + QA_BIAS_OFF, qpos, hi, my, mx, p.sy, p.sx);
     auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
 #pragma unroll
@@ -331,7 +376,12 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
     const LoadVTransposed<DB, decltype(v_step)> load_v(lane_t, v_step);
     f32x16 o[DB];
     float sum;
+#if defined(QA_LAB) && QA_LAB >= 1
+    sum = 1.f;
+    for (int db = 0; db < DB; ++db) for (int e = 0; e < 16; ++e) o[db][e] = __builtin_bit_cast(float, __builtin_bit_cast(u32x4, qf[e & 3])[db]);
+#else
     attention_sweep<NQ, KS, DB, HAS_BIAS>(logits, load_k, load_v, [](int) {}, qf, o, sum);
+#endif
     const uint32_t tok = (uint32_t)un.b * (uint32_t)(H * W) + (window_wraps(un) ? token_in_image(un, qpos) : window_base(un) + q_rel);
     // the next unit's projection bias: requested ahead of the output stores (vector memory operations complete in order)
     u32x2 bq_next[QA_FN];
@@ -351,13 +401,15 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
   // ---- flat pipeline over (unit, k-tile), ping-pong between the two wave groups: see gemm_persistent.hip.  Per
   // k-tile j the slots M0 | C0 | M1 | C1; a memory slot reads the fragments of half a k-tile (8 + 3 ds_read_b128) and
   // issues loads (M0: the wave's 4 of A[j + 1]; M1: its 3 of W[j + 2]), a compute slot issues 24 MFMAs; group 1 runs
-  // one slot behind group 0.  Waits: group 0 at the end of its C1(j) until only its 3 loads of W[j + 2] are
-  // outstanding; group 1 for W[j + 1] at the end of its M1(j) (4 + 3 newer loads) and for A[j + 1] at the end of its
-  // C1(j).  Two k-tiles of a unit differ.  The last one issues no A load (the stage it would fill carries Q first;
-  // the load follows in attend()): group 1's wait in M1 then counts 3 newer loads.  The first one of every unit but
-  // the workgroup's first also issues the 2 loads of the head's bias 4-vectors, after its A loads: group 1's wait in
-  // M1 counts 4 + 2 + 3 newer loads, the wait at the end of C1 leaves 2 + 3 outstanding.
-  const int total = n_my * KT;
+  // one slot behind group 0.  Waits: at the end of M1(j) for W[j + 1] (4 + 3 newer loads), at the end of C1(j) until
+  // only the 3 loads of W[j + 2] are outstanding.
+  // A compute slot here is 24 MFMAs = 384 cycles, a quarter shorter than the GEMM's: the memory slot of the other
+  // group has to fit under it, so the k-tiles of a unit come in four kinds, each compiled as straight-line code of its
+  // own without run-time decisions: FIRST also issues the 2 loads of the head's bias 4-vectors behind its A loads
+  // (waits: 4 + 2 + 3 newer loads in M1, 2 + 3 outstanding after C1); MIDDLE; NEXT_TO_LAST, whose W loads open the next
+  // unit's weight rows; LAST, which issues no A load (the stage it would fill carries Q first: attend() issues it)
+  // and whose M1 wait therefore counts 3 newer loads.  In the workgroup's last unit the last two kinds wait for all.
+  enum { FIRST = 0, MIDDLE = 1, NEXT_TO_LAST = 2, LAST = 3 };
   la_set_unit();
   lw_set_unit();
   issue_bias(decode(0).head);
@@ -366,20 +418,20 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
   issue_w();
   __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   __syncthreads();
-  int j = 0, sa = 0, sw = 0;
+  int sa = 0, sw = 0;
   for (int r = 0; r < n_my; ++r) {
     if (grp == 1) __builtin_amdgcn_s_barrier();
-    int sw_last = 0;
+    const bool has_next = r + 1 < n_my;
+    const bool with_bias = HAS_BIAS && r > 0;  // the first unit's bias came in with the prologue
     const int cur_head = decode(r).head;
-    for (int kt = 0; kt < KT; ++kt, ++j) {
+    int sw_last = 0;
+    auto k_tile = [&](auto kind_c) {
+      constexpr int KIND = decltype(kind_c)::value;
       const unsigned char* s_a = smem + sa * QA_A_BYTES;
       const unsigned char* s_w = smem + QA_W_OFF + sw * QA_W_BYTES;
       sw_last = sw;
       sa ^= 1;
-      if (++sw == 3) sw = 0;
-      const bool more = j + 2 < total;
-      const bool last_kt = kt + 1 == KT;
-      const bool bias_kt = HAS_BIAS && kt == 0 && r > 0;
+      sw = sw == 2 ? 0 : sw + 1;
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         bf16x8 af[QA_FM], bfr[QA_FN];
@@ -389,17 +441,25 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
         for (int jn = 0; jn < QA_FN; ++jn) bfr[jn] = *reinterpret_cast<const bf16x8*>(s_w + b_roff[half] + jn * 16 * 128);
         __builtin_amdgcn_sched_barrier(0);
         if (half == 0) {
-          if (!last_kt) issue_a();
-          if (bias_kt) issue_bias(cur_head);
+          if (KIND != LAST) issue_a_same_unit();
+          if (KIND == FIRST && with_bias) issue_bias(cur_head);
         } else {
-          issue_w();
+          if (KIND == FIRST || KIND == MIDDLE) {
+            issue_w_same_unit();
+          } else {  // the next unit's first two k-tiles of W (nothing once the list has ended)
+            if (KIND == NEXT_TO_LAST) lw_next_unit();
+            issue_w();
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (half == 0 || grp == 0) __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
-        else if (!more) __builtin_amdgcn_s_waitcnt(WAIT_ALL);
-        else if (last_kt) __builtin_amdgcn_s_waitcnt(WAIT_VM3_LGKM0);
-        else if (bias_kt) __builtin_amdgcn_s_waitcnt(WAIT_VM9_LGKM0);
-        else __builtin_amdgcn_s_waitcnt(WAIT_VM7_LGKM0);
+        if (half == 0) __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
+        else if (KIND == MIDDLE) __builtin_amdgcn_s_waitcnt(WAIT_VM7_LGKM0);
+        else if (KIND == FIRST) {
+          if (with_bias) __builtin_amdgcn_s_waitcnt(WAIT_VM9_LGKM0);
+          else __builtin_amdgcn_s_waitcnt(WAIT_VM7_LGKM0);
+        } else if (!has_next) __builtin_amdgcn_s_waitcnt(WAIT_ALL);
+        else if (KIND == NEXT_TO_LAST) __builtin_amdgcn_s_waitcnt(WAIT_VM7_LGKM0);
+        else __builtin_amdgcn_s_waitcnt(WAIT_VM3_LGKM0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -409,21 +469,28 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
             acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[jn], af[i], acc[i][jn], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (half == 1) {
-          if (!more) __builtin_amdgcn_s_waitcnt(WAIT_VM0);
-          else if (bias_kt) __builtin_amdgcn_s_waitcnt(WAIT_VM5);
+          if (KIND == MIDDLE) __builtin_amdgcn_s_waitcnt(WAIT_VM3);
+          else if (KIND == FIRST) {
+            if (with_bias) __builtin_amdgcn_s_waitcnt(WAIT_VM5);
+            else __builtin_amdgcn_s_waitcnt(WAIT_VM3);
+          } else if (!has_next) __builtin_amdgcn_s_waitcnt(WAIT_VM0);
           else __builtin_amdgcn_s_waitcnt(WAIT_VM3);
         }
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       }
-    }
+    };
+    k_tile(std::integral_constant<int, FIRST>{});
+    for (int kt = 1; kt < KT - 2; ++kt) k_tile(std::integral_constant<int, MIDDLE>{});
+    k_tile(std::integral_constant<int, NEXT_TO_LAST>{});
+    k_tile(std::integral_constant<int, LAST>{});
     if (grp == 0) __builtin_amdgcn_s_barrier();
     attend(r, sw_last);
   }
 }
 
 bool qkv_attention_supported(int ws_y, int ws_x, int head_dim, int K, int64_t tokens_per_image) {
-  return ws_y == QA_WS && ws_x == QA_WS && head_dim == QA_HD && K > 0 && K % 128 == 0 &&
+  return ws_y == QA_WS && ws_x == QA_WS && head_dim == QA_HD && K >= 256 && K % 128 == 0 &&
          tokens_per_image * K * 2 < (int64_t)0xFFFFFFF0u;
 }
 
@@ -459,9 +526,8 @@ hipError_t qkv_attention_launch(const void* y, const void* w, const void* bias, 
   p.use_mask = use_mask;
   p.q_scale = scale * 1.4426950408889634f;
   p.n_win = B * p.nWy * p.nWx;
-  p.total_units = p.n_win * heads;
-  p.per_xcd = (p.total_units + 7) / 8;
-  p.bpx = p.per_xcd < 32 ? p.per_xcd : 32;
+  const int max_seq = ((p.n_win + QA_GM - 1) / QA_GM + 7) / 8 * QA_GM * heads;  // units of the XCD with the most groups
+  p.bpx = max_seq < 32 ? max_seq : 32;
   const dim3 grid(8 * p.bpx), block(QA_NT);
   if (bias4) hipLaunchKernelGGL(qkv_window_attention_kernel<true>, grid, block, QA_SMEM, stream, p);
   else hipLaunchKernelGGL(qkv_window_attention_kernel<false>, grid, block, QA_SMEM, stream, p);

@@ -412,14 +412,15 @@ window_attention_dma_kernel(AttnParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Persistent form of the kernel above: one workgroup per CU walks a contiguous range of (head, window) units, one
-// wave per 32-query group, with two K / V buffer sets in LDS.  While the waves compute unit i from one set, the load
-// unit fills the other with unit i + 1 (buffer_load ... lds costs the waves 8 instructions each and no registers), so
-// the HBM stream and the arithmetic overlap inside one workgroup instead of depending on how two independent
-// workgroups on a CU happen to interleave.  One workgroup barrier per unit: a wave passes it when its share of unit
-// i + 1 has landed; everyone having passed it means unit i's buffers are free for unit i + 2.
-// Units are ordered head-major, so a workgroup's consecutive units share the head and its relative-position bias
-// column in LDS is rebuilt only when the head changes.
+// Persistent form of the kernel above: one workgroup per CU walks every gridDim-th (head, window) unit, one wave per
+// 32-query group, with two K / V buffer sets in LDS.  While the waves compute unit i from one set, the load unit fills
+// the other with the workgroup's next unit (buffer_load ... lds costs the waves 8 instructions each and no
+// registers), so the HBM stream and the arithmetic overlap inside one workgroup instead of depending on how two
+// independent workgroups on a CU happen to interleave.  One workgroup barrier per unit: a wave passes it when its
+// share of the next unit has landed; everyone having passed it means the current unit's buffers are free for the unit
+// after the next.  Units are numbered head-major and the stride is far smaller than the windows of one head, so a
+// workgroup's consecutive units nearly always share the head: its relative-position bias column in LDS is rebuilt
+// only when the head changes.
 template <int WS_Y, int WS_X, bool HAS_BIAS>
 struct AttnPersistCfg {
   static constexpr int L = WS_Y * WS_X;
@@ -435,7 +436,7 @@ constexpr int attn_persist_threads(int ws_y, int ws_x) { return ((ws_y * ws_x + 
 
 template <int WS_Y, int WS_X, bool HAS_BIAS>
 __global__ void __launch_bounds__(attn_persist_threads(WS_Y, WS_X))
-window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
+window_attention_persist_kernel(AttnParams p, int n_units) {
   using Cfg = AttnPersistCfg<WS_Y, WS_X, HAS_BIAS>;
   constexpr int HD = 64, KS = 4, DB = 2;
   constexpr int L = Cfg::L, NQ = Cfg::NQ, LPAD = Cfg::LPAD, NT = Cfg::NT, TBL = Cfg::TBL, KVB = Cfg::KV_BYTES;
@@ -459,16 +460,17 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
   const int wpi = p.nWy * p.nWx;
   const int n_win = p.B * wpi;
 
-  const int u_begin = blockIdx.x * units_per_wg;
-  int u_end = u_begin + units_per_wg;
-  if (u_end > n_units) u_end = n_units;
-  if (u_begin >= u_end) return;
+  const int u_begin = blockIdx.x, u_step = gridDim.x;
+  if (u_begin >= n_units) return;
 
   const uint32_t plane_bytes = (uint32_t)p.B * (uint32_t)(H * W) * ld_qkv * 2u;  // < 2^32, checked by the caller
   const int rsub = lane >> 3, pc = lane & 7;
 
-  // A unit = (head, batch entry, window row, window column), walked window-fastest; everything about it is
-  // workgroup-uniform and lives in scalar registers.  The successor of a unit follows by carries, without a division.
+  // A unit = (head, batch entry, window row, window column), numbered window-fastest; everything about it is
+  // workgroup-uniform and lives in scalar registers.  A workgroup takes the units u_begin, u_begin + u_step, ...: the
+  // windows on the wrapped border of a shifted grid (a whole window row; their mask arithmetic makes them the slow
+  // ones) are then spread over all workgroups instead of filling the ranges of a few.  The successor of a unit
+  // follows by adding the digits of u_step with carries, without a division.
   struct Unit { int head, b, wy, wx; };
   auto decode = [&](int u) {
     Unit r;
@@ -480,17 +482,18 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
     r.wx = wrem - r.wy * p.nWx;
     return r;
   };
+  const Unit step = decode(u_step);
   auto successor = [&](Unit r) {
-    if (++r.wx == p.nWx) {
-      r.wx = 0;
-      if (++r.wy == p.nWy) {
-        r.wy = 0;
-        if (++r.b == p.B) {
-          r.b = 0;
-          ++r.head;
-        }
-      }
-    }
+    r.wx += step.wx;
+    int carry = r.wx >= p.nWx;
+    r.wx -= carry ? p.nWx : 0;
+    r.wy += step.wy + carry;
+    carry = r.wy >= p.nWy;
+    r.wy -= carry ? p.nWy : 0;
+    r.b += step.b + carry;
+    carry = r.b >= p.B;
+    r.b -= carry ? p.B : 0;
+    r.head += step.head + carry;
     return r;
   };
   // Token row of window position (iy, ix): away from the wrapped border (every window of an un-shifted grid, all but
@@ -590,11 +593,12 @@ window_attention_persist_kernel(AttnParams p, int units_per_wg, int n_units) {
 #pragma unroll
   for (int s2 = 0; s2 < KS; ++s2) q_nxt[s2] = q_cur[s2];
 
-  for (int u = u_begin; u < u_end; ++u) {
-    const int set = (u - u_begin) & 1;
-    const bool more = u + 1 < u_end;
+  int set = 1;
+  for (int u = u_begin; u < n_units; u += u_step) {
+    set ^= 1;
+    const bool more = u + u_step < n_units;
     const Unit nxt = successor(cur);
-    if (HAS_BIAS && cur.head != bias_head) {  // workgroup-uniform and rare: the range crosses into the next head
+    if (HAS_BIAS && cur.head != bias_head) {  // workgroup-uniform and rare: the walk crosses into the next head
       __syncthreads();
       build_bias(cur.head);
       bias_head = cur.head;
@@ -714,10 +718,8 @@ static hipError_t launch_attn(const AttnParams& p, hipStream_t stream) {
       (int64_t)p.B * p.H * p.W * p.tok_stride * 2 < (int64_t)0xFFFFFFF0u) {
     if (grid >= 2 * (int64_t)g_attn_cus) {  // enough units for every CU to stream a few: the persistent form
       using P = AttnPersistCfg<WS_Y, WS_X, HAS_BIAS>;
-      const int per = (int)((grid + g_attn_cus - 1) / g_attn_cus);
-      const int wgs = (int)((grid + per - 1) / per);
-      hipLaunchKernelGGL((window_attention_persist_kernel<WS_Y, WS_X, HAS_BIAS>), dim3((unsigned)wgs), dim3(P::NT), P::SMEM,
-                         stream, p, per, (int)grid);
+      hipLaunchKernelGGL((window_attention_persist_kernel<WS_Y, WS_X, HAS_BIAS>), dim3((unsigned)g_attn_cus), dim3(P::NT), P::SMEM,
+                         stream, p, (int)grid);
       return hipGetLastError();
     }
     using D = AttnDmaCfg<WS_Y, WS_X, HAS_BIAS>;

@@ -187,7 +187,7 @@ def window_attention(qkv: torch.Tensor, B: int, image_shape: Tuple[int, int], he
 def qkv_attention_supported(K: int, heads: int, head_dim: int, window_size, image_shape) -> bool:
     """Whether the fused to_qkv + window attention kernel takes this shape (16x16 windows, head_dim 64, K % 128 == 0)."""
     H, W = image_shape
-    return (tuple(window_size) == (16, 16) and head_dim == 64 and K % 128 == 0 and H % 16 == 0 and W % 16 == 0
+    return (tuple(window_size) == (16, 16) and head_dim == 64 and K % 128 == 0 and K >= 256 and H % 16 == 0 and W % 16 == 0
             and H * W * K * 2 < 0xFFFFFFF0 and 3 * heads * head_dim * K * 2 < 2 ** 31)
 
 

@@ -114,7 +114,7 @@ int aeris_window_attention_heads_fwd(const void* qkv_planes, void* out, const vo
  * the same softmax(q k^T + bias + mask) v as aeris_window_attention_heads_fwd from on-chip memory.  Replaces
  * model.py:299-307 (+ the swin_shift calls at model.py:471-475 on one device): the same result as aeris_gemm_heads_fwd
  * (with q_scale) followed by aeris_window_attention_heads_fwd (q_prescaled), bit for bit.
- * Built for 16x16 windows, head_dim 64, K % 128 == 0, H*W*K*2 < 2^32; anything else: AERIS_EUNSUPPORTED. */
+ * Built for 16x16 windows, head_dim 64, K % 128 == 0, K >= 256, H*W*K*2 < 2^32; anything else: AERIS_EUNSUPPORTED. */
 int64_t aeris_qkv_attention_bias_bytes(int heads, int ws_y, int ws_x);
 int aeris_qkv_attention_prepare_bias(const void* bias_table, int heads, int ws_y, int ws_x, void* out, void* stream);
 int aeris_qkv_window_attention_fwd(const void* y, const void* w, const void* qkv_bias, const void* bias4, void* out,

@@ -387,7 +387,7 @@ FUSED_CASES = [
     (1, 160, 160, 24, 1536, 8, True, True),    # configs[3] widths: 24 k-tiles, 2400 units
     (1, 160, 160, 24, 256, 0, False, False),   # 4 k-tiles, no bias anywhere: accumulators start at a literal zero
     (2, 96, 160, 6, 384, 8, True, False),      # two batch entries, 120 windows x 6 heads
-    (1, 48, 80, 3, 128, 8, True, True),        # 15 windows (the last group of 4 is short), 2 k-tiles, 45 units < 256 workgroups
+    (1, 48, 80, 3, 256, 8, True, True),        # 15 windows (the last group of 4 is short), 4 k-tiles (the fewest), 45 units < 256 workgroups
     (1, 32, 32, 2, 640, 8, True, True),        # every window on the wrapped border; 8 units
 ]
 
@@ -437,6 +437,7 @@ def test_fused_qkv_window_attention_rejects_other_shapes(pkg, cuda):
     assert not ops.qkv_attention_supported(1536, 24, 64, (12, 12), (180, 360))
     assert not ops.qkv_attention_supported(1536, 12, 128, (16, 16), (160, 160))
     assert not ops.qkv_attention_supported(1472, 24, 64, (16, 16), (160, 160))  # K % 128
+    assert not ops.qkv_attention_supported(128, 2, 64, (16, 16), (160, 160))  # fewer than 4 k-tiles
     y = torch.zeros(144 * 4, 128, dtype=torch.bfloat16, device=cuda)
     w = torch.zeros(3 * 64, 128, dtype=torch.bfloat16, device=cuda)
     with pytest.raises(pkg.AerisError) as e:

@@ -122,12 +122,13 @@ def test_argument_validation_needs_no_gpu(pkg):
     qa, qb, qp = lib.aeris_qkv_window_attention_fwd, lib.aeris_qkv_attention_bias_bytes, lib.aeris_qkv_attention_prepare_bias
     assert qb(24, 16, 16) == 24 * 961 * 16 and qb(24, 12, 12) == 0 and qb(0, 16, 16) == 0
     assert qp(None, 24, 16, 16, p16, None) == L.EINVAL and qp(p16, 24, 8, 8, p16, None) == L.EUNSUPPORTED
-    okq = (p16, p16, None, None, p16, 1, 32, 32, 2, 64, 128, 16, 16, 8, 8, 1, 0.125, None)
+    okq = (p16, p16, None, None, p16, 1, 32, 32, 2, 64, 256, 16, 16, 8, 8, 1, 0.125, None)
     def withq(i, v):
         a = list(okq); a[i] = v; return a
     assert qa(*withq(0, None)) == L.EINVAL and qa(*withq(4, None)) == L.EINVAL  # y / out NULL
     assert qa(*withq(2, p16 + 2)) == L.EINVAL  # projection bias not 8-byte aligned
-    assert qa(*withq(9, 128)) == L.EUNSUPPORTED and qa(*withq(10, 192)) == L.EUNSUPPORTED  # head_dim, K % 128
+    assert qa(*withq(9, 128)) == L.EUNSUPPORTED and qa(*withq(10, 320)) == L.EUNSUPPORTED  # head_dim, K % 128
+    assert qa(*withq(10, 128)) == L.EUNSUPPORTED  # fewer than four k-tiles
     assert qa(*withq(11, 32)) == L.EUNSUPPORTED  # 32x16 windows
     assert "aeris_gemm_heads_fwd" in L.last_error()  # the message names the two-kernel path to use instead
     assert qa(*withq(13, 16)) == L.EINVAL  # shift outside the window

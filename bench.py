@@ -204,6 +204,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--no-fused-compare", action="store_true",
+                    help="skip the second timing of the step with to_qkv + window attention as ONE kernel")
     ap.add_argument("--ensemble", type=int, default=4, help="config4: ensemble members (batch)")
     ap.add_argument("--sampler-steps", type=int, default=10, help="config4: sampler steps (2n-1 denoiser calls per forecast step)")
     args = ap.parse_args()
@@ -259,13 +261,42 @@ def main():
             model(x, t)
         rec = pkg.ops.profile_end()
 
+        # the same step with to_qkv + window attention as ONE kernel (q, k, v never in HBM) where the block shape allows it:
+        # timed beside the default so that the choice of the default is a measurement of this run
+        fused_rec, fused_elapsed = None, None
+        attn_mods = [m for m in model.modules() if isinstance(m, pkg.model.Attention)]
+        if not args.no_fused_compare and attn_mods:
+            was = [m.fuse_qkv for m in attn_mods]
+            for m in attn_mods:
+                m.fuse_qkv = not m.fuse_qkv
+            try:
+                model(x, t)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    model(x, t)
+                torch.cuda.synchronize()
+                fused_elapsed = time.perf_counter() - t0
+                pkg.ops.profile_begin()
+                for _ in range(args.steps):
+                    model(x, t)
+                fused_rec = pkg.ops.profile_end()
+            finally:
+                for m, v in zip(attn_mods, was):
+                    m.fuse_qkv = v
+
     ms_per_step = elapsed / args.steps * 1e3
-    agg = {}
-    for tag, work, unit, ms in rec:
-        a = agg.setdefault(tag, {"launches": 0, "work": 0.0, "ms": 0.0, "unit": unit})
-        a["launches"] += 1
-        a["work"] += work
-        a["ms"] += ms
+
+    def aggregate(records):
+        out = {}
+        for tag, work, unit, ms in records:
+            a = out.setdefault(tag, {"launches": 0, "work": 0.0, "ms": 0.0, "unit": unit})
+            a["launches"] += 1
+            a["work"] += work
+            a["ms"] += ms
+        return out
+
+    agg = aggregate(rec)
     kernels = {}
     for tag, a in agg.items():
         rate = a["work"] / (a["ms"] * 1e-3)
@@ -311,6 +342,38 @@ def main():
                               "spec (LayerNorm, scale/shift modulation, rel-pos bias, shift mask, GELU MLP, biases)")},
         "roofline": roofline, "kernels": kernels, "output_finite": finite,
     }
+    if fused_rec is not None:
+        other = aggregate(fused_rec)
+        default_fused = "qkv_window_attention" in agg
+        both = other if not default_fused else agg      # the run in which the one-kernel form was used
+        pair = agg if not default_fused else other      # the run with the to_qkv GEMM and the attention kernel apart
+        if "qkv_window_attention" in both:
+            a = both["qkv_window_attention"]
+            one_ms = a["ms"] / a["launches"]
+            tfl = a["work"] / (a["ms"] * 1e-3) / 1e12
+            inner = wl["heads"] * wl["head_dim"]
+            attn_flop = 4.0 * S * wl["window"] ** 2 * inner
+            byts = 2.0 * S * wl["dim"] + 2.0 * S * inner + 2.0 * 3 * inner * wl["dim"]  # y in, o out, the weight once
+            two = {}
+            for tag in ("gemm_256x256_none_bf16_plain", "window_attention"):
+                if tag in pair:
+                    two[tag] = pair[tag]["ms"] / pair[tag]["launches"]
+            result["qkv_attention_one_kernel"] = {
+                "kernel": "qkv_window_attention_kernel<HAS_BIAS> (to_qkv GEMM, q scaling, window attention; q, k, v stay in LDS)",
+                "is_default": default_fused, "launches_per_step": a["launches"] // args.steps, "avg_ms": one_ms,
+                "tflops": tfl, "frac_mfma_peak": tfl / PEAK_BF16_TFLOPS,
+                "attention_part_tflops_beside_separate_gemm_time": None,
+                "hbm_bytes_algorithmic": byts, "hbm_gbs_algorithmic": byts / (one_ms * 1e-3) / 1e9,
+                "frac_hbm_peak": byts / (one_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                "two_kernels_avg_ms": two, "two_kernels_sum_ms": sum(two.values()) if len(two) == 2 else None,
+                "ms_per_step_with_one_kernel": (fused_elapsed if not default_fused else elapsed) / args.steps * 1e3,
+                "ms_per_step_with_two_kernels": (elapsed if not default_fused else fused_elapsed) / args.steps * 1e3,
+            }
+            if len(two) == 2:
+                rest = one_ms - two["gemm_256x256_none_bf16_plain"]
+                if rest > 0:
+                    result["qkv_attention_one_kernel"]["attention_part_tflops_beside_separate_gemm_time"] = \
+                        attn_flop / (rest * 1e-3) / 1e12
     if not args.no_cpu_baseline:
         result["cpu_baseline"], result["parity"] = cpu_baseline_and_parity(pkg, torch, wl, model, args.cpu_rows, dev, res_dt)
         result["gpu_over_cpu"] = result["value"] / result["cpu_baseline"]["value"]

@@ -166,9 +166,11 @@ class RoPE2D(nn.Module):
 
 
 # Whether ``Attention`` runs the to_qkv projection inside the attention kernel where that kernel exists (16x16 windows,
-# head_dim 64, dim % 128 == 0) instead of as a GEMM that writes q, k, v to HBM for a separate attention kernel.  Both
-# paths compute the same bits; this picks the faster one as measured on the benchmark's shape.
-FUSE_QKV_ATTENTION = False
+# head_dim 64, dim % 128 == 0 and >= 256) instead of as a GEMM that writes q, k, v to HBM for a separate attention
+# kernel.  Both paths compute the same bits.  Inside the benchmark's denoiser step the one-kernel form is the faster of
+# the two (13.96-13.99 ms against 11.5-11.7 + 2.67-2.68 ms per block, 0.5-0.8 % of the step; bench.py times the step both
+# ways in every run), so it is the default; every other shape takes the pair.
+FUSE_QKV_ATTENTION = True
 
 
 class Attention(nn.Module):

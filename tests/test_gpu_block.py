@@ -132,6 +132,32 @@ def test_small_model_parity(pkg, cuda, preset, res_dt):
     assert rel_l2(out, ref) <= 1e-2
 
 
+def test_model_output_does_not_depend_on_the_attention_path(pkg, cuda):
+    """``Attention.fuse_qkv`` chooses between the to_qkv GEMM + attention kernel pair and the one kernel that keeps
+    q, k, v on the chip; both compute the same bits wherever the pair's GEMM is the 256x256-tile kernel (same MFMA shape
+    and k order; the grid here is large enough for that), so the whole model's output is bit-identical either way
+    (shifted and unshifted blocks, bias table, mask, linear biases, batch 2)."""
+    geo = dict(MODEL_GEO, image_shape=(96, 128))
+    cfg = OracleConfig.spec(mod_ways=2, n_layers=6, in_channels=138, out_channels=69, **geo)
+    assert pkg.ops.gemm_uses_big_tiles(2 * 96 * 128, 3 * cfg.heads * cfg.head_dim)
+    sd = oracle.init_model_weights(cfg, 13, nontrivial=True)
+    model = make_model(pkg, cfg, sd, cuda, torch.float32, "spec")
+    attn = [m for m in model.modules() if isinstance(m, pkg.model.Attention)]
+    assert attn and all(m.fuse_qkv == pkg.model.FUSE_QKV_ATTENTION for m in attn)
+    assert all(pkg.ops.qkv_attention_supported(cfg.dim, m.heads, m.head_dim, m.window_size, m.image_shape) for m in attn)
+    g = torch.Generator().manual_seed(23)
+    x, dt = torch.randn(2, 96 * 128, 138, generator=g).to(cuda), torch.tensor([0.7]).to(cuda)
+    outs = {}
+    for fuse in (True, False):
+        for m in attn:
+            m.fuse_qkv = fuse
+        pkg.ops.profile_begin()
+        outs[fuse] = model(x, dt).clone()
+        tags = {r[0] for r in pkg.ops.profile_end()}
+        assert ("qkv_window_attention" in tags) == fuse and ("window_attention" in tags) == (not fuse), tags
+    assert torch.equal(outs[True], outs[False])
+
+
 def test_reference_window_model_parity(pkg, cuda):
     """The reference's own window geometry (60 x 60 windows of 3600 tokens, head_dim 128, model.py:22-27; preset
     "ref": RMSNorm, 3-way modulation, SwiGLU, no bias / mask) on a 120 x 180 grid: input stage -> 2 layers (the

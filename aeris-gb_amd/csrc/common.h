@@ -81,6 +81,8 @@ __device__ __forceinline__ void lds_dma_load16(const lds_dma_rsrc& rsrc, uint32_
 // result registers must pass through lds_tr_wait() (s_waitcnt lgkmcnt(0)) before anything reads them.  ("memory"
 // keeps the compiler from moving LDS accesses of its own across the read; its own lgkmcnt waits stay correct, LDS
 // operations return in order and extra outstanding ones only make a counted wait stricter.)
+// Nor does the compiler keep such a read away from registers that a running MFMA is still writing (see the sweep in
+// attention_sweep.h).  Both rules are checked on the emitted assembly by every build (asm_check.py, run by build.py).
 __device__ __forceinline__ uint32_t lds_byte_address(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }

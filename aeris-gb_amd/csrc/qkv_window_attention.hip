@@ -359,8 +359,13 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
     __builtin_amdgcn_sched_barrier(0);
     // 3. the sweep
     // (wave-uniform, and said so: the mask arithmetic must stay behind a scalar branch that all but the border windows skip)
+#ifdef QA_LAB_MASK_EVERY  // timing experiment: every QA_LAB_MASK_EVERY-th unit of a workgroup takes the mask path
+    const bool my = __builtin_amdgcn_readfirstlane((int)(p.use_mask && (r_done % QA_LAB_MASK_EVERY) == 0)) != 0;
+    const bool mx = false;
+#else
     const bool my = __builtin_amdgcn_readfirstlane((int)(p.use_mask && p.sy > 0 && un.wy == p.nWy - 1)) != 0;
     const bool mx = __builtin_amdgcn_readfirstlane((int)(p.use_mask && p.sx > 0 && un.wx == p.nWx - 1)) != 0;
+#endif
     const WindowLogits<QA_WS, QA_WS, HAS_BIAS> logits(smem + QA_BIAS_OFF, qpos, hi, my, mx, p.sy, p.sx);
     auto load_k = [&](int kb, bf16x8 (&f)[KS]) {
 #pragma unroll

@@ -169,9 +169,20 @@ def cpu_baseline_and_parity(pkg, torch, wl, model, rows, dev, residual_dtype):
         got = strip(x.to(dev), t.to(dev)).float().cpu()
         warm = torch.randn(512, 512)
         (warm @ warm).sum().item()  # spin up the thread pool
+        import threading
+        done = threading.Event()
+
+        def heartbeat():  # the oracle prints nothing for up to minutes (the 60x60-window workload); say that the run is alive
+            while not done.wait(45.0):
+                print(f"bench.py: CPU oracle running, {time.perf_counter() - t0:.0f} s", file=sys.stderr, flush=True)
+
         t0 = time.perf_counter()
-        want = oracle.model_forward(cfg, sd, x, t)
-        t_strip = time.perf_counter() - t0
+        threading.Thread(target=heartbeat, daemon=True).start()
+        try:
+            want = oracle.model_forward(cfg, sd, x, t)
+            t_strip = time.perf_counter() - t0
+        finally:
+            done.set()
     del strip
     diff = (got.double() - want.double())
     parity = {"rel_l2": float(diff.norm() / want.double().norm()), "max_abs": float(diff.abs().max()),
@@ -265,7 +276,8 @@ def main():
         # the same step with to_qkv + window attention as ONE kernel (q, k, v never in HBM) where the block shape allows it:
         # timed beside the default so that the choice of the default is a measurement of this run
         fused_rec, fused_elapsed = None, None
-        attn_mods = [m for m in model.modules() if isinstance(m, pkg.model.Attention)]
+        attn_mods = [m for m in model.modules() if isinstance(m, pkg.model.Attention) and
+                     pkg.ops.qkv_attention_supported(wl["dim"], m.heads, m.head_dim, m.window_size, m.image_shape)]
         if not args.no_fused_compare and attn_mods:
             was = [m.fuse_qkv for m in attn_mods]
             for m in attn_mods:

@@ -90,6 +90,7 @@ struct WindowLogits {
   static constexpr int L = WS_Y * WS_X, LPAD = (L + 31) / 32 * 32, TBL = (2 * WS_Y - 1) * (2 * WS_X - 1);
   static constexpr float MASK_NEG = -100.0f * 1.4426950408889634f;  // the additive -100, in the exp2 domain
   const unsigned char* sB;
+  const unsigned char* sB_lane;  // sB + (sp + 4 hi) * 16: the lane's part of every bias vector address
   int sp, hi;
   bool my, mx;
   int ry_q, rx_q, sy, sx;
@@ -100,6 +101,7 @@ struct WindowLogits {
       : sB(bias_lds), hi(hi_), my(my_), mx(mx_), sy(sy_), sx(sx_) {
     const int qiy = qpos / WS_X, qix = qpos % WS_X;
     sp = (TBL - 1) - (qiy + WS_Y - 1) * (2 * WS_X - 1) - qix - (WS_X - 1);
+    sB_lane = sB + (sp + 4 * hi) * 16;
     ry_q = my ? (qiy < WS_Y - sy ? 1 : 2) : 0;
     rx_q = mx ? (qix < WS_X - sx ? 1 : 2) : 0;
   }
@@ -108,10 +110,19 @@ struct WindowLogits {
     for (int g = 0; g < 4; ++g) {
       f32x4 bv = {0.f, 0.f, 0.f, 0.f};
       if (HAS_BIAS) {
-        const int key0 = kb * 32 + g * 8 + hi * 4;
-        const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
-        const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
-        bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+        if (WS_X % 8 == 0 && LPAD == L) {
+          // the lane's 4 keys start at column (8-aligned part) + 4 hi of their window row and never cross into the next
+          // row: the index is the lane's own part, sp + 4 hi, plus a part that is a constant once kb is one (the
+          // unrolled sweep): a per-lane base address and an immediate offset, no arithmetic per key group
+          const int base = kb * 32 + g * 8;
+          const int qt0 = (base / WS_X) * (2 * WS_X - 1) + (base % WS_X);
+          bv = *reinterpret_cast<const f32x4*>(sB_lane + qt0 * 16);
+        } else {
+          const int key0 = kb * 32 + g * 8 + hi * 4;
+          const int kk = ((LPAD == L) || key0 < L) ? key0 : 0;
+          const int qt = (kk / WS_X) * (2 * WS_X - 1) + (kk % WS_X);
+          bv = *reinterpret_cast<const f32x4*>(sB + (sp + qt) * 16);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) a[g * 4 + i] = bv[i];

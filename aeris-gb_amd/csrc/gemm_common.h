@@ -27,6 +27,9 @@ struct GemmParams {
   int total_tiles;
   int per_xcd;  // tiles in one XCD's contiguous chunk
   int bpx;      // workgroups per XCD
+  // ceil(2^40 / (tiles per L2 group)): t / group size = (t * m_gsz) >> 40 for t < 2^24 (a tile is decoded several
+  // times per tile and wave; a true division is some 25 vector ALU operations each time)
+  uint64_t m_gsz;
   int act;
   int res_dtype;  // -1 none, AERIS_BF16, AERIS_F32
   int c_dtype;

@@ -77,10 +77,11 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   auto decode = [&](int r, int& tile_m, int& tile_n) {
     const int t = chunk0 + r * p.bpx + slot;
     const int gsz = GM * p.tiles_n;
-    const int grp = t / gsz, within = t - grp * gsz;
+    const int grp = (int)(((uint64_t)(uint32_t)t * p.m_gsz) >> 40), within = t - grp * gsz;
     int gm = p.tiles_m - grp * GM;
     if (gm > GM) gm = GM;
-    tile_n = within / gm;
+    static_assert(GM == 4, "the shift below");
+    tile_n = gm == GM ? within >> 2 : within / gm;  // only the last group of row panels can be short
     tile_m = grp * GM + (within - tile_n * gm);
   };
 
@@ -756,6 +757,8 @@ hipError_t gemm_persistent_launch(const GemmParams& p0, hipStream_t stream) {
   p.total_tiles = p.tiles_m * p.tiles_n;
   p.per_xcd = (p.total_tiles + 7) / 8;
   p.bpx = p.per_xcd < 32 ? p.per_xcd : 32;  // 32 CUs per XCD, one workgroup each
+  if (p.total_tiles >= (1 << 24)) return hipErrorInvalidValue;  // the range of the multiply-shift division
+  p.m_gsz = (((uint64_t)1 << 40) + (uint64_t)(GM * p.tiles_n) - 1) / (uint64_t)(GM * p.tiles_n);
   dim3 grid(8 * p.bpx), block(NT);
   const bool f32 = p.c_dtype == AERIS_F32;
   const bool plain = !p.gate && p.res_dtype < 0;

@@ -63,7 +63,11 @@ struct QkvAttnParams {
   int use_mask;
   float q_scale;          // softmax scale times log2(e)
   int n_win, bpx;         // windows (B * nWy * nWx); workgroups per XCD
+  // ceil(2^40 / d) for d = units per group, windows per image, windows per row: n / d = (n * m) >> 40 for n < 2^24.
+  // A unit is decoded several times per unit and wave; as true divisions that was 40 % of the kernel's vector ALU work.
+  uint64_t m_gsz, m_wpi, m_nwx;
 };
+__device__ __forceinline__ int div_by_magic(int n, uint64_t m) { return (int)(((uint64_t)(uint32_t)n * m) >> 40); }
 }  // namespace
 
 // R4[head][s][e] = table[TBL - 1 - (s + e)][head] * log2(e) for s + e < TBL, else 0: the layout WindowLogits reads
@@ -105,17 +109,18 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
   struct Unit { int head, b, wy, wx; };
   auto decode = [&](int r) {
     const int t = r * p.bpx + slot;
-    const int lg = t / gsz, within = t - lg * gsz;
+    const int lg = div_by_magic(t, p.m_gsz), within = t - lg * gsz;
     const int g = lg * 8 + xcd;
     int gm = p.n_win - g * QA_GM;
     if (gm > QA_GM) gm = QA_GM;
     Unit u;
-    u.head = within / gm;
+    static_assert(QA_GM == 4, "the shift below");
+    u.head = gm == QA_GM ? within >> 2 : within / gm;  // only the very last group can be short
     const int win = g * QA_GM + (within - u.head * gm);
     const int wpi = p.nWy * p.nWx;
-    u.b = win / wpi;
+    u.b = div_by_magic(win, p.m_wpi);
     const int wrem = win - u.b * wpi;
-    u.wy = wrem / p.nWx;
+    u.wy = div_by_magic(wrem, p.m_nwx);
     u.wx = wrem - u.wy * p.nWx;
     return u;
   };
@@ -532,6 +537,11 @@ hipError_t qkv_attention_launch(const void* y, const void* w, const void* bias, 
   p.q_scale = scale * 1.4426950408889634f;
   p.n_win = B * p.nWy * p.nWx;
   const int max_seq = ((p.n_win + QA_GM - 1) / QA_GM + 7) / 8 * QA_GM * heads;  // units of the XCD with the most groups
+  if ((int64_t)p.n_win * heads >= (1 << 24)) return hipErrorInvalidValue;  // the range of div_by_magic
+  auto magic = [](int d) { return (((uint64_t)1 << 40) + (uint64_t)d - 1) / (uint64_t)d; };
+  p.m_gsz = magic(QA_GM * heads);
+  p.m_wpi = magic(p.nWy * p.nWx);
+  p.m_nwx = magic(p.nWx);
   p.bpx = max_seq < 32 ? max_seq : 32;
   const dim3 grid(8 * p.bpx), block(QA_NT);
   if (bias4) hipLaunchKernelGGL(qkv_window_attention_kernel<true>, grid, block, QA_SMEM, stream, p);

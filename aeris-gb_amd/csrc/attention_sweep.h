@@ -130,16 +130,33 @@ struct WindowLogits {
   }
   __device__ __forceinline__ void mask_block(int kb, f32x16& a) const {
     if (my || mx) {
+      if (WS_X % 8 == 0 && LPAD == L) {
+        // as in init_acc: the lane's 4 keys of a group lie in one window row, whose number is a constant once kb is; what
+        // depends on the lane is whether column (8-aligned part) + 4 hi + i has wrapped around, one compare per key
+        const int h4 = 4 * hi;
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < 4; ++g) {
+          const int base = kb * 32 + g * 8;
+          const int kiy = base / WS_X, cx0 = base % WS_X;
+          const bool ydiff = my && ((kiy < WS_Y - sy) != (ry_q == 1));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = kb * 32 + g * 8 + hi * 4 + i;
-          const int kiy = key / WS_X, kix = key % WS_X;
-          const int ry_k = my ? (kiy < WS_Y - sy ? 1 : 2) : 0;
-          const int rx_k = mx ? (kix < WS_X - sx ? 1 : 2) : 0;
-          if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
+          for (int i = 0; i < 4; ++i) {
+            const bool xdiff = mx && ((h4 < WS_X - sx - i - cx0) != (rx_q == 1));
+            if (ydiff || xdiff) a[g * 4 + i] += MASK_NEG;
+          }
         }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = kb * 32 + g * 8 + hi * 4 + i;
+            const int kiy = key / WS_X, kix = key % WS_X;
+            const int ry_k = my ? (kiy < WS_Y - sy ? 1 : 2) : 0;
+            const int rx_k = mx ? (kix < WS_X - sx ? 1 : 2) : 0;
+            if (ry_k != ry_q || rx_k != rx_q) a[g * 4 + i] += MASK_NEG;
+          }
+      }
     }
     if (LPAD != L) {
 #pragma unroll

@@ -110,7 +110,10 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   __amdgpu_buffer_rsrc_t rs_a = rs_w;
   int la_r = 0, la_kt = 0, la_stage = 0;  // A stream
   auto la_set_tile = [&]() {
-    if (la_r >= n_my) return;
+    if (la_r >= n_my) {  // past the end of the list: a descriptor without records, the loads fetch nothing
+      rs_a = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, 0, 0x00020000);
+      return;
+    }
     int tile_m, tile_n;
     decode(la_r, tile_m, tile_n);
     const int64_t m0 = (int64_t)tile_m * BM;
@@ -118,26 +121,32 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     if (rows > BM) rows = BM;
     rs_a = __builtin_amdgcn_make_buffer_rsrc((void*)(p.A + m0 * K), 0, (int)(rows * K * 2), 0x00020000);
   };
+  // Always 4 loads, also past the end of the list (into stages nobody reads any more, from a descriptor without
+  // records): the number of loads in flight at any point of the k-loop is then the same for every k-tile, and no wait
+  // has to be chosen at run time.
   auto issue_a = [&]() {
-    if (la_r < n_my) {
-      unsigned char* sd = smem + la_stage * A_BYTES + wave_u * 4096;
-      const uint32_t so = (uint32_t)(wave_u * 32) * (uint32_t)(K * 2) + (uint32_t)la_kt * (BK * 2);
+    unsigned char* sd = smem + la_stage * A_BYTES + wave_u * 4096;
+    const uint32_t so = (uint32_t)(wave_u * 32) * (uint32_t)(K * 2) + (uint32_t)la_kt * (BK * 2);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(sd + i * 1024), 16, ld_voff[i & 1],
-                                                 so + (uint32_t)(i * 8) * (uint32_t)(K * 2), 0, 0);
-      la_stage ^= 1;
-      if (++la_kt == KT) {
-        la_kt = 0;
-        ++la_r;
-        la_set_tile();
-      }
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(sd + i * 1024), 16, ld_voff[i & 1],
+                                               so + (uint32_t)(i * 8) * (uint32_t)(K * 2), 0, 0);
+    la_stage ^= 1;
+    if (++la_kt == KT) {
+      la_kt = 0;
+      ++la_r;
+      la_set_tile();
     }
   };
   uint32_t lw_row = 0;  // W row of the first of this wave's 32 rows of the tile
   int lw_r = 0, lw_kt = 0, lw_stage = 0;  // W stream
+  __amdgpu_buffer_rsrc_t rs_wc = rs_w;  // the W stream's descriptor: rs_w, or one without records past the end of the list
   auto lw_set_tile = [&]() {
-    if (lw_r >= n_my) return;
+    if (lw_r >= n_my) {
+      rs_wc = __builtin_amdgcn_make_buffer_rsrc((void*)p.W, 0, 0, 0x00020000);
+      lw_row = 0;
+      return;
+    }
     int tile_m, tile_n;
     decode(lw_r, tile_m, tile_n);
     const int n0 = tile_n * BN_OUT;
@@ -146,19 +155,17 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     else lw_row = (uint32_t)(n0 + wave_u * 32);
   };
   auto issue_w = [&]() {
-    if (lw_r < n_my) {
-      unsigned char* sd = smem + B_OFF + lw_stage * B_BYTES + wave_u * 4096;
-      const uint32_t so = lw_row * (uint32_t)(K * 2) + (uint32_t)lw_kt * (BK * 2);
+    unsigned char* sd = smem + B_OFF + lw_stage * B_BYTES + wave_u * 4096;
+    const uint32_t so = lw_row * (uint32_t)(K * 2) + (uint32_t)lw_kt * (BK * 2);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(sd + i * 1024), 16, ld_voff[i & 1],
-                                                 so + (uint32_t)(i * 8) * (uint32_t)(K * 2), 0, 0);
-      if (++lw_stage == B_STAGES) lw_stage = 0;
-      if (++lw_kt == KT) {
-        lw_kt = 0;
-        ++lw_r;
-        lw_set_tile();
-      }
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_wc, (lds_ptr)(sd + i * 1024), 16, ld_voff[i & 1],
+                                               so + (uint32_t)(i * 8) * (uint32_t)(K * 2), 0, 0);
+    if (++lw_stage == B_STAGES) lw_stage = 0;
+    if (++lw_kt == KT) {
+      lw_kt = 0;
+      ++lw_r;
+      lw_set_tile();
     }
   };
 
@@ -682,7 +689,6 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       const unsigned char* s_w = smem + B_OFF + sw * B_BYTES;
       sa ^= 1;
       if (++sw == B_STAGES) sw = 0;
-      const bool more = j + 2 < total;  // W[j+2] (and so A[j+1]) exist
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         // ---- memory slot: LDS reads first (queued, non-blocking), then the loads
@@ -695,9 +701,10 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         if (half == 0) issue_a();
         else issue_w();
         __builtin_amdgcn_sched_barrier(0);
-        if (half == 0 || grp == 0) __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
-        else if (more) __builtin_amdgcn_s_waitcnt(WAIT_VM8_LGKM0);
-        else __builtin_amdgcn_s_waitcnt(WAIT_ALL);
+        // (group 0 needs its rows of W[j+1] only one slot later and could do without the vmcnt part here; waiting in both
+        // groups costs nothing - those loads are a k-tile old - and spares a decision per slot)
+        if (half == 0) __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
+        else __builtin_amdgcn_s_waitcnt(WAIT_VM8_LGKM0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         // ---- compute slot
@@ -707,10 +714,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           for (int jn = 0; jn < FN; ++jn)
             acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[jn], af[i], acc[i][jn], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (half == 1) {
-          if (more) __builtin_amdgcn_s_waitcnt(WAIT_VM4);
-          else __builtin_amdgcn_s_waitcnt(WAIT_VM0);
-        }
+        if (half == 1) __builtin_amdgcn_s_waitcnt(WAIT_VM4);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       }

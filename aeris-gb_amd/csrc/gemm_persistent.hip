@@ -665,12 +665,12 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   // anything the epilogue has issued in between only makes a wait more conservative): group 0 reads A[j+1] and
   // W[j+1] in slot 4j+4.  Each wave of group 0 waits at the end of its C1(j) until only its 4 loads of W[j+2] are
   // outstanding; each wave of group 1 waits for its rows of W[j+1] at the end of its M1(j) (slot 4j+3; 8 newer
-  // loads) and for its rows of A[j+1] at the end of its C1(j).  At the end of the list, where fewer loads follow,
-  // the wait is for all.
+  // loads) and for its rows of A[j+1] at the end of its C1(j).  Both groups take both waits (for group 0 the first
+  // one is early, for loads a k-tile old), and the streams keep issuing past the end of the list, so the waits are
+  // the same constants in every k-tile: nothing is decided at run time between a barrier and the next MFMAs.
   // A slot ends in a bare s_barrier: the fences of __syncthreads() would make every wave wait for all of its
   // outstanding loads into LDS.  What a barrier has to order is stated explicitly with s_waitcnt.
-  constexpr int WAIT_LGKM0 = 0xC07F, WAIT_VM0 = 0x0F70, WAIT_VM4 = 0x0F74, WAIT_VM8_LGKM0 = 0x0078, WAIT_ALL = 0x0070;
-  const int total = n_my * KT;
+  constexpr int WAIT_LGKM0 = 0xC07F, WAIT_VM0 = 0x0F70, WAIT_VM4 = 0x0F74, WAIT_VM8_LGKM0 = 0x0078;
   la_set_tile();
   lw_set_tile();
   issue_a();
@@ -678,13 +678,13 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   issue_w();
   __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   __syncthreads();
-  int j = 0, sa = 0, sw = 0;  // position in the flat list of k-tiles, its A and W stages
+  int sa = 0, sw = 0;  // the A and W stages of the k-tile at hand
   for (int r = 0; r < n_my; ++r) {
     // Group 1 runs one slot behind group 0.  The offset is set up anew for every tile (group 1 waits one slot
     // here, group 0 one slot before its epilogue), so that both groups run their epilogues at the same time:
     // with the epilogues one slot apart, each would hold up the other group at a barrier.
     if (grp == 1) __builtin_amdgcn_s_barrier();
-    for (int kt = 0; kt < KT; ++kt, ++j) {
+    for (int kt = 0; kt < KT; ++kt) {
       const unsigned char* s_a = smem + sa * A_BYTES;
       const unsigned char* s_w = smem + B_OFF + sw * B_BYTES;
       sa ^= 1;

@@ -190,7 +190,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     decode(r, tile_m, tile_n);
     return tile_n * BN_OUT + (wave_u % WN) * (SWIGLU ? 32 : BN / WN);
   };
-  auto load_bias = [&](int r, u32x2 (&bq)[FN]) {
+  auto load_bias = [&](int r, u32x2 (&bq)[FN], int q) {  // q: lane >> 4, from the caller (the epilogue passes its own copy)
     const int n_wave = wave_col0(r);
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
@@ -210,9 +210,12 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   };
   {
     u32x2 bq[FN];
-    load_bias(0, bq);
+    load_bias(0, bq, q);
     init_acc(bq);
   }
+
+  // s_waitcnt immediates: vmcnt in bits 3:0 (and 15:14), expcnt in 6:4 (7 = no wait), lgkmcnt in 11:8 (15 = no wait)
+  constexpr int WAIT_LGKM0 = 0xC07F, WAIT_VM0 = 0x0F70, WAIT_VM4 = 0x0F74, WAIT_VM8_LGKM0 = 0x0078;
 
   // ---- epilogue of the tile whose accumulators are complete.
   // Vector memory operations of a wave complete in order, so a wait for a load also waits for every store issued
@@ -340,6 +343,13 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     // its 64-byte rows; +2 %).  For the other forms this was slower (qkv -4 %, proj -5 %: 64-byte row pieces), although
     // gate and residual are then applied in fp32 before the only rounding.
     const bool interior_direct = SWIGLU && PLAIN && !OUT_F32 && rows_left == BM / WM && n_wave + 32 <= N;
+    // Every path ends in a wait of its own.  Nothing that writes a register may be pending when the k-loop is entered:
+    // the compiler would guard the fragment registers with a wait for all vector memory operations inside the loop,
+    // on every k-tile, which cuts the lead of the W loads to one slot.  The first k-tile needs the oldest loads at once
+    // anyway.  Stores write no register: the straight-line paths end with 4 of them behind their last load (the next
+    // tile's bias) and leave those to drain under the first slots of the next tile, whose first counted wait (end of
+    // M1(0)) covers them.  The wait has to stand inside the path: behind the join the compiler no longer knows that the
+    // operations left outstanding are stores, and puts a wait for all of them into the k-loop.
     if (interior_direct) {
       // No staging: after a swap between lane rows (v_permlane16_swap on the registers of column fragments 2m and
       // 2m + 1) lane (l15, q) owns 8 consecutive columns, 32 m + 16 (q & 1) + 8 (q >> 1) .., of row 16 i + l15: four
@@ -353,7 +363,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       }
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
-        if (i + 1 == FM && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+        if (i + 1 == FM && r_done + 1 < n_my) load_bias(r_done + 1, bq_next, q);
 #pragma unroll
         for (int m = 0; m < NP; ++m) {
           float a[4], b[4];
@@ -364,7 +374,8 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           *reinterpret_cast<u32x4*>(c_lane[m] + (int64_t)__mul24(i * 16 + l15, rs24) * 2) = u32x4{rx[0], ry[0], rx[1], ry[1]};
         }
       }
-    }     else if (interior) {
+      __builtin_amdgcn_s_waitcnt(WAIT_VM0);
+    } else if (interior) {
       const int n = n_wave + rch * 8;
       unsigned char* const c_lane =
           reinterpret_cast<unsigned char*>(p.C) + (m_base * c_row_stride(p) + c_col_off(p, n)) * 2;
@@ -407,11 +418,12 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_wave_barrier();
         // the next loads go ahead of the stores below
         if (RES_BF16 && i + 2 < FM / 2) load_res(i + 2);
-        if (i + 1 == FM / 2 && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+        if (i + 1 == FM / 2 && r_done + 1 < n_my) load_bias(r_done + 1, bq_next, q);
 #pragma unroll
         for (int it = 0; it < 4; ++it)
           *reinterpret_cast<u32x4*>(c_lane + (int64_t)__mul24(i * 32 + rrow + 8 * it, rs24) * 2) = out[it];
       }
+      __builtin_amdgcn_s_waitcnt(WAIT_VM4);  // the 4 stores of the last block may still be on their way
     } else if (!OUT_F32) {
       // stage 2 (bf16 C): a whole 32 x 64 (SwiGLU: 32 x 32) block through LDS, rows of 128 B, chunk-swizzled; it
       // is read back as 16-byte chunks, 8 lanes per row, and C / residual are accessed as full row segments
@@ -497,7 +509,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         if (i + 1 < FM / 2) {
           if (res_dtype >= 0) load_res(i + 1);  // ahead of the stores below
         } else if (r_done + 1 < n_my) {
-          load_bias(r_done + 1, bq_next);
+          load_bias(r_done + 1, bq_next, q);
         }
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -509,6 +521,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           }
         }
       }
+      __builtin_amdgcn_s_waitcnt(WAIT_VM0);
     } else if (RES_F32 && ACT != AERIS_ACT_SWIGLU && rows_left == BM / WM && n_wave + BN / WN <= N && !gate_per_lane) {
       // Interior tiles with f32 C and an f32 residual: the staging of the general f32 path below (units of 32 rows x
       // 32 columns through the wave's 4 KB), as straight-line code without per-lane conditions, the residual rows
@@ -558,11 +571,12 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (u + 2 < UNITS) load_res(u + 2);  // ahead of the stores below
-        if (u + 1 == UNITS && r_done + 1 < n_my) load_bias(r_done + 1, bq_next);
+        if (u + 1 == UNITS && r_done + 1 < n_my) load_bias(r_done + 1, bq_next, q);
 #pragma unroll
         for (int it = 0; it < 4; ++it)
           *reinterpret_cast<f32x4*>(c_lane + ((int64_t)__mul24(i * 32 + rrow + 8 * it, ld24) + j * 32) * 4) = out[it];
       }
+      __builtin_amdgcn_s_waitcnt(WAIT_VM4);  // the 4 stores of the last unit may still be on their way
     } else {
       // stage 2 (f32 C): units of 32 rows x 32 columns (2 x 2 fragments), rows of 128 B (32 floats), 4 floats per
       // lane and row
@@ -636,7 +650,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
         if (u + 1 < UNITS) {
           if (p.res_dtype >= 0) load_res(u + 1);  // ahead of the stores below
         } else if (r_done + 1 < n_my) {
-          load_bias(r_done + 1, bq_next);
+          load_bias(r_done + 1, bq_next, q);
         }
         const int n = unit_col(u);
         unsigned char* const c_lane =
@@ -647,6 +661,7 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
           if (r < rows_left && n < N) *reinterpret_cast<f32x4*>(c_lane + (int64_t)__mul24(r, rs24) * 4) = out[it];
         }
       }
+      __builtin_amdgcn_s_waitcnt(WAIT_VM0);
     }
     if (r_done + 1 < n_my) init_acc(bq_next);
   };
@@ -670,7 +685,6 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
   // the same constants in every k-tile: nothing is decided at run time between a barrier and the next MFMAs.
   // A slot ends in a bare s_barrier: the fences of __syncthreads() would make every wave wait for all of its
   // outstanding loads into LDS.  What a barrier has to order is stated explicitly with s_waitcnt.
-  constexpr int WAIT_LGKM0 = 0xC07F, WAIT_VM0 = 0x0F70, WAIT_VM4 = 0x0F74, WAIT_VM8_LGKM0 = 0x0078;
   la_set_tile();
   lw_set_tile();
   issue_a();
@@ -721,10 +735,6 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
     }
     if (grp == 0) __builtin_amdgcn_s_barrier();
     epilogue(r);  // leaves the accumulators at the bias of the next tile
-    // Nothing that writes a register may be pending when the k-loop is entered: the compiler would guard the
-    // fragment registers with a wait for all vector memory operations inside the loop, on every k-tile, which
-    // cuts the lead of the W loads to one slot.  The first k-tile needs the oldest loads at once anyway.
-    __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   }
 }
 

@@ -291,7 +291,7 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
 
   // s_waitcnt immediates: vmcnt in bits 3:0 (and 15:14), expcnt in 6:4 (7 = no wait), lgkmcnt in 11:8 (15 = no wait)
   constexpr int WAIT_LGKM0 = 0xC07F, WAIT_VM0 = 0x0F70, WAIT_VM3 = 0x0F73, WAIT_VM5 = 0x0F75, WAIT_VM3_LGKM0 = 0x0073,
-                WAIT_VM7_LGKM0 = 0x0077, WAIT_VM9_LGKM0 = 0x0079, WAIT_ALL = 0x0070;
+                WAIT_VM7_LGKM0 = 0x0077, WAIT_VM9_LGKM0 = 0x0079, WAIT_VM4_LGKM0 = 0x0074, WAIT_ALL = 0x0070;
 
   // ---- attention on the finished tile (in place of a GEMM epilogue)
   auto attend = [&](int r_done, int sw_last) {
@@ -403,7 +403,10 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
     // 4. K, V and the bias slot are free again once every wave is through; and every wave's rows of the next unit's
     // first k-tile of A (issued above) have landed before any wave reads them.  Nothing that writes a register is
     // pending when the k-loop is entered again (see gemm_persistent.hip).
-    __builtin_amdgcn_s_waitcnt(WAIT_ALL);
+    // The 4 output stores (the last vector memory operations of this phase; they write no register) drain under the
+    // next unit's first slots, whose first counted wait covers them.
+    static_assert(DB * 2 == 4, "the wait below counts the output stores");
+    __builtin_amdgcn_s_waitcnt(WAIT_VM4_LGKM0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };

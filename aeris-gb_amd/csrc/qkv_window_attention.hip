@@ -307,7 +307,6 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
     {  // timing only: the main loop alone (the accumulators are folded into one store so that they stay live)
       f32x4 t = {0.f, 0.f, 0.f, 0.f};
       for (int i = 0; i < QA_FM; ++i) for (int j = 0; j < QA_FN; ++j) t += acc[i][j];
-      la_next_unit();
       issue_a();
       *reinterpret_cast<f32x4*>(p.out + ((uint64_t)un.b * (uint32_t)(H * W) + window_base(un) + q_rel) * (uint32_t)inner + un.head * QA_HD + hi * 8) = t;
       u32x2 bq0[QA_FN];
@@ -324,25 +323,33 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
     unsigned char* const sV1 = smem + QA_SPARE_OFF;                   // V rows 192..255
     // 1. q (times scale * log2 e), k, v -> bf16 -> LDS.  A lane holds 4 consecutive d of one token per fragment: half
     // of a 16-byte chunk of the token's row; Q and K rows are chunk-swizzled by (row >> 1) & 7, V rows by 2 (row & 3).
+    // The position of row fragment i is that of fragment 0 plus 16 i, which leaves both swizzles as they are: the
+    // address of fragment i is the address of fragment 0 plus 2048 i, an immediate offset of the write, so a column
+    // fragment needs one address (written out per fragment, the address arithmetic was nine tenths of this phase).
+    // V rows 192..255 live in the spare area: for the upper wave group that is the fragments i >= 4.
+    {
+      const int row0 = wm * (QA_BM / QA_WM) + l15;
+      const uint32_t qk_row = (uint32_t)(row0 >> 1) * 256u, qk_hi = (uint32_t)((row0 & 1) << 3), qk_sw = (uint32_t)((row0 >> 1) & 7);
+      const uint32_t v_row = (uint32_t)row0 * 128u, v_sw = (uint32_t)(2 * (row0 & 3));
 #pragma unroll
-    for (int j = 0; j < QA_FN; ++j) {
-      const int col = wn * 48 + j * 16;       // wave-uniform: first tile column of the fragment
-      const int part = col >> 6, d0 = (col & 63) + q4 * 4;
-      const int chunk = d0 >> 3, half = (d0 >> 2) & 1;
-#pragma unroll
-      for (int i = 0; i < QA_FM; ++i) {
-        const int row = wm * (QA_BM / QA_WM) + i * 16 + l15;  // window position
-        f32x4 v = acc[i][j];
-        if (part == 0) v *= p.q_scale;
-        const u32x2 w2 = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        unsigned char* dst;
+      for (int j = 0; j < QA_FN; ++j) {
+        const int col = wn * 48 + j * 16;       // wave-uniform: first tile column of the fragment
+        const int part = col >> 6, d0 = (col & 63) + q4 * 4;
+        const uint32_t chunk = (uint32_t)(d0 >> 3), half8 = (uint32_t)(((d0 >> 2) & 1) * 8);
+        const float sc = part == 0 ? p.q_scale : 1.0f;  // a scalar: times 1 is exact, and cheaper than selecting per value
+        unsigned char *dst_lo, *dst_hi;  // fragment i goes to (i < 4 ? dst_lo : dst_hi) + 2048 i
         if (part == 2) {
-          unsigned char* base = row < 192 ? sV0 + row * 128 : sV1 + (row - 192) * 128;
-          dst = base + ((chunk ^ (2 * (row & 3))) << 4) + half * 8;
+          const uint32_t a = v_row + ((chunk ^ v_sw) << 4) + half8;
+          dst_lo = sV0 + a;
+          dst_hi = wm == 0 ? dst_lo : sV1 + a - 192 * 128;
         } else {
-          dst = (part == 0 ? sQ : sK) + (row >> 1) * 256 + (((((row & 1) << 3) | chunk) ^ ((row >> 1) & 7)) << 4) + half * 8;
+          dst_lo = dst_hi = (part == 0 ? sQ : sK) + qk_row + (((qk_hi | chunk) ^ qk_sw) << 4) + half8;
         }
-        *reinterpret_cast<u32x2*>(dst) = w2;
+#pragma unroll
+        for (int i = 0; i < QA_FM; ++i) {
+          const f32x4 v = acc[i][j] * sc;
+          *reinterpret_cast<u32x2*>((i < QA_FM / 2 ? dst_lo : dst_hi) + i * 2048) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        }
       }
     }
     __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
@@ -356,9 +363,10 @@ __global__ void __launch_bounds__(QA_NT) qkv_window_attention_kernel(QkvAttnPara
       qf[s2] = *reinterpret_cast<const bf16x8*>(sQ + (row >> 1) * 256 + (((((row & 1) << 3) | chunk) ^ ((row >> 1) & 7)) << 4));
     }
     __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
-    __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    // every wave has its Q: A0 may be refilled with the next unit's first k-tile (held back in the main loop)
+    // This wave has its Q, and the 4 KB of A0 that its own loads fill are exactly the 16 position pairs it has just read
+    // (positions 32 wave .. 32 wave + 31, read by no other wave): it refills them with its rows of the next unit's first
+    // k-tile (held back in the main loop) without waiting for the other waves.
     la_next_unit();
     issue_a();
     __builtin_amdgcn_sched_barrier(0);

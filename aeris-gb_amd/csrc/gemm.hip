@@ -278,7 +278,8 @@ hipError_t gemm_launch(const void* A, const void* W, void* C, const void* bias, 
   const int bn_out = swiglu ? 128 : 256;
   const bool big = (M >= 256) && (N % bn_out == 0 || N >= 4 * bn_out) &&
                    ((M + 255) / 256) * ((N + bn_out - 1) / bn_out) >= 256 &&
-                   ((M + 255) / 256) * ((N + bn_out - 1) / bn_out) < (int64_t(1) << 24);  // the persistent kernel's tile numbering
+                   ((M + 255) / 256) * ((N + bn_out - 1) / bn_out) < (int64_t(1) << 24) &&  // the persistent kernel's tile numbering
+                   M + 512 < (int64_t(1) << 31);  // ... and its 32-bit row numbers
   // vector epilogue (8 / 16 byte accesses to C and the residual) needs 4-element alignment of every row
   const bool vec = (split || (ldc & 3) == 0) && ((N & 3) == 0);
   if (!vec) return swiglu ? launch_gemm<128, 128, 2, 2, true, false>(p, stream) : launch_gemm<128, 128, 2, 2, false, false>(p, stream);

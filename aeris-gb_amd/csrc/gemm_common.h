@@ -30,6 +30,11 @@ struct GemmParams {
   // ceil(2^40 / (tiles per L2 group)): t / group size = (t * m_gsz) >> 40 for t < 2^24 (a tile is decoded several
   // times per tile and wave; a true division is some 25 vector ALU operations each time)
   uint64_t m_gsz;
+  // row / rows_per_batch = (row * rpb_magic) >> rpb_shift, exact for row, rows_per_batch < 2^31 (magic = ceil(2^shift /
+  // rows_per_batch), shift = 31 + ceil(log2 rows_per_batch)): the batch entry of a tile's rows, for the per-batch gate.
+  // As 64-bit divisions these were some 400 scalar instructions per tile and wave, through the CU's one scalar unit.
+  uint32_t rpb_magic;
+  int rpb_shift;
   int act;
   int res_dtype;  // -1 none, AERIS_BF16, AERIS_F32
   int c_dtype;

@@ -272,7 +272,8 @@ __global__ void __launch_bounds__(NT) gemm_bf16_nt_persistent_kernel(GemmParams 
       } else {
         int64_t last = m_base + BM / WM - 1;
         if (last > p.M - 1) last = p.M - 1;
-        const int64_t b0 = m_base / p.rows_per_batch, b1 = last / p.rows_per_batch;
+        const int64_t b0 = (int64_t)(((uint64_t)(uint32_t)m_base * p.rpb_magic) >> p.rpb_shift);
+        const int64_t b1 = (int64_t)(((uint64_t)(uint32_t)last * p.rpb_magic) >> p.rpb_shift);
         if (b0 == b1) {
           gate_tile = p.gate + b0 * p.gate_batch_stride;
         } else {
@@ -773,6 +774,15 @@ hipError_t gemm_persistent_launch(const GemmParams& p0, hipStream_t stream) {
   p.bpx = p.per_xcd < 32 ? p.per_xcd : 32;  // 32 CUs per XCD, one workgroup each
   if (p.total_tiles >= (1 << 24)) return hipErrorInvalidValue;  // the range of the multiply-shift division
   p.m_gsz = (((uint64_t)1 << 40) + (uint64_t)(GM * p.tiles_n) - 1) / (uint64_t)(GM * p.tiles_n);
+  // rows of a tile (first row of a wave group, at most tiles_m * 256 + 128) and rows_per_batch below 2^31
+  if ((int64_t)p.tiles_m * BM + BM >= (int64_t(1) << 31) || p.rows_per_batch <= 0 || p.rows_per_batch >= (int64_t(1) << 31))
+    return hipErrorInvalidValue;
+  {
+    int lg = 0;
+    while (((int64_t)1 << lg) < p.rows_per_batch) ++lg;
+    p.rpb_shift = 31 + lg;
+    p.rpb_magic = (uint32_t)((((uint64_t)1 << p.rpb_shift) + (uint64_t)p.rows_per_batch - 1) / (uint64_t)p.rows_per_batch);
+  }
   dim3 grid(8 * p.bpx), block(NT);
   const bool f32 = p.c_dtype == AERIS_F32;
   const bool plain = !p.gate && p.res_dtype < 0;

@@ -14,6 +14,13 @@ registers, so two properties that it guarantees for its own instructions have to
    destination registers overlap the read's (the compiler may hand registers it can prove dead to the read while the
    MFMA that last wrote them is still running; the MFMA's late write then replaces what the read returned).
 
+3. counted wait behind loads into LDS: a ``s_waitcnt vmcnt(N) lgkmcnt(0)`` with N > 0 stands where a kernel waits for
+   its ``buffer_load ... lds`` loads but lets the N stores issued after them drain later (vector memory operations
+   complete in order, so "at most N outstanding" covers everything older than the N youngest).  That only holds if N
+   vector memory instructions really follow the loads on every path: the N youngest ones before the wait must be
+   stores in the wait's own basic block (no label in between), so that no path can skip them.  (Checked wherever a
+   store is among them; the counted waits of the k-loops stand between loads only.)
+
     python aeris-gb_amd/asm_check.py file.s [...]      # exit status 1 if a rule is broken
 
 ``check_text`` is what build.py runs on the device assembly of every source that contains such reads.
@@ -25,6 +32,8 @@ import sys
 
 MFMA_WINDOW = 24  # instructions; an MFMA of these kernels is done at most 16 passes after it issued
 _REG = re.compile(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b")
+_TAIL_WAIT = re.compile(r"^s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)$")
+_VMEM = ("global_", "buffer_", "flat_", "scratch_")
 _KERNEL_LABEL = re.compile(r"^(_Z\w+):")
 
 
@@ -45,6 +54,7 @@ def check_text(asm: str):
     problems, n_reads = [], 0
     kernel, pending, recent_mfma, n_ins = None, {}, [], 0
     labels_in_window, window_id = {}, 0
+    block_vmem = []  # vector memory instructions of the current basic block, in order
     for ln, raw in enumerate(asm.splitlines(), 1):
         m = _KERNEL_LABEL.match(raw)
         if m:
@@ -57,10 +67,22 @@ def check_text(asm: str):
         if t.endswith(":"):
             if pending:
                 labels_in_window[t[:-1]] = window_id
+            block_vmem = []
             continue
         if t.startswith("."):
             continue
         n_ins += 1
+        if t.startswith(_VMEM):
+            block_vmem.append(t)
+        m = _TAIL_WAIT.match(t)
+        if m and int(m.group(1)) > 0:
+            n = int(m.group(1))
+            tail = block_vmem[-n:]
+            is_store = [x.split()[0].startswith(("global_store", "buffer_store")) for x in tail]
+            # (a counted wait with no store among the youngest operations is one of the k-loops' waits between loads)
+            if any(is_store) and (len(tail) < n or not all(is_store)):
+                problems.append(f"{kernel} line {ln}: `{t}` is not preceded by {n} stores in its basic block "
+                                f"(found {[x.split()[0] for x in tail]})")
         if t.startswith(("s_cbranch", "s_branch")) and t.split()[-1] in labels_in_window:
             if not pending or labels_in_window[t.split()[-1]] != window_id:
                 problems.append(f"{kernel} line {ln}: `{t}` jumps back into the window of a transposing read")

@@ -91,3 +91,27 @@ def test_state_does_not_leak_between_kernels():
     two = kernel(["ds_read_b64_tr_b16 v[10:11], v3 offset:0", "s_waitcnt lgkmcnt(0)"]) + \
         kernel(["v_mov_b32_e32 v4, v10"]).replace("testEv", "test2Ev")
     assert asm_check.check_text(two) == ([], 1)
+
+
+def test_counted_wait_behind_stores():
+    ok = ["buffer_load_dwordx4 v2, s[44:47], s7 offen lds",
+          "global_load_dwordx2 v[8:9], v[4:5], off",
+          "global_store_dwordx4 v[40:41], v[20:23], off",
+          "global_store_dwordx4 v[40:41], v[4:7], off offset:64",
+          "s_waitcnt vmcnt(1)",                       # the compiler's own wait for the load
+          "global_store_dwordx4 v[40:41], v[4:7], off offset:96",
+          "global_store_dwordx4 v[40:41], v[20:23], off offset:32",
+          "s_waitcnt vmcnt(4) lgkmcnt(0)",
+          "s_barrier"]
+    assert asm_check.check_text(kernel(ok))[0] == []
+    # one of the four youngest operations is a load: the wait could leave an LDS load pending
+    bad = list(ok)
+    bad[2], bad[1] = ok[1], ok[2]
+    problems, _ = asm_check.check_text(kernel(bad))
+    assert len(problems) == 1 and "not preceded by 4 stores" in problems[0]
+    # a label among them: a path could reach the wait without having issued all four
+    skip = ok[:6] + [".LBB0_9:"] + ok[6:]
+    problems, _ = asm_check.check_text(kernel(skip))
+    assert len(problems) == 1 and "not preceded by 4 stores" in problems[0]
+    # the main loops' counted waits (no lgkmcnt(0) ... or vmcnt(0)) are not meant
+    assert asm_check.check_text(kernel(["buffer_load_dwordx4 v2, s[44:47], s7 offen lds", "s_waitcnt vmcnt(0) lgkmcnt(0)"]))[0] == []

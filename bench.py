@@ -27,10 +27,10 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Bytes that crossed the L2 <-> fabric boundary per launch at the config3 workload (average over the launches of
 # one step), from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a 1 GiB copy kernel; the summary
 # with the commands is profiles/denoiser_step_config3_pmc_traffic.txt.  Not measurable from inside this script.
-PMC_TRAFFIC_BYTES = {"config3": {"gemm_256x256_none_f32": 30.734e9 + 6.375e9, "gemm_256x256_none_bf16_plain": 33.418e9 + 9.555e9,
-                                 "gemm_256x256_gelu_bf16_plain": 31.394e9 + 12.740e9, "window_attention": 9.572e9 + 3.187e9,
-                                 "qkv_window_attention": 36.867e9 + 3.185e9,
-                                 "norm_modulate": 6.463e9 + 3.185e9, "output_stage": 6.383e9 + 0.286e9}}
+PMC_TRAFFIC_BYTES = {"config3": {"gemm_256x256_none_f32": 30.169e9 + 6.373e9, "gemm_256x256_none_bf16_plain": 40.273e9 + 9.555e9,
+                                 "gemm_256x256_gelu_bf16_plain": 31.556e9 + 12.740e9, "window_attention": 9.573e9 + 3.187e9,
+                                 "qkv_window_attention": 31.338e9 + 3.185e9,
+                                 "norm_modulate": 6.463e9 + 3.185e9, "output_stage": 6.384e9 + 0.286e9}}
 
 WORKLOADS = {
     # name: grid, dim, heads, head_dim, window, mlp, blocks, in/out channels
